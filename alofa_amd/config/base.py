@@ -76,5 +76,13 @@ class ModelConfig:
         """config.json content that ``from_dict`` reads back to an equal config."""
         raise NotImplementedError
 
+    def wants_shapes(self) -> bool:
+        """Whether some size of the model is given by a tensor's shape rather than by config.json."""
+        return False
+
+    def sized_by(self, shapes: dict) -> "ModelConfig":
+        """The configuration with such sizes filled in from ``shapes`` (tensor name -> shape)."""
+        return self
+
     def spec(self) -> ModelSpec:
         raise NotImplementedError

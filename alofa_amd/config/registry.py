@@ -1,4 +1,4 @@
-"""One registry from the architecture's name (config.json ``architectures[0]``)
+"""One registry from the architecture's name (config.json ``architectures[0]``, or ``architecture``)
 to its configuration class. The reference wires its single architecture in
 directly (src/alofa/engine/executor.mojo:61-80); the registry is this
 engine's own."""
@@ -42,6 +42,8 @@ def _reject_duplicate_keys(pairs):
 
 def config_from_dict(raw: dict, where: str = "<dict>") -> ModelConfig:
     archs = raw.get("architectures")
+    if archs is None and isinstance(raw.get("architecture"), str):      # (some designs name their one architecture plainly)
+        archs = [raw["architecture"]]
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
         raise AlofaError("invalid_argument", "config.json names no architecture", f"config={where}")
     return config_class(archs[0]).from_dict(raw, where)
@@ -59,4 +61,8 @@ def load_config(model_dir) -> ModelConfig:
         raise AlofaError("parse", "config.json is not valid JSON", f"path={path} reason={e}") from None
     if not isinstance(raw, dict):
         raise AlofaError("parse", "config.json must hold one object", f"path={path}")
-    return config_from_dict(raw, str(path))
+    cfg = config_from_dict(raw, str(path))
+    if cfg.wants_shapes():      # sizes that config.json leaves to the tensors' shapes (read from the files' headers only)
+        from ..weights.loader import weight_files
+        cfg = cfg.sized_by({n: tuple(f.shape(n)) for n, f in weight_files(model_dir).items()})
+    return cfg

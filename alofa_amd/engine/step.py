@@ -88,7 +88,8 @@ class StepContext:
         self._slots: list = []
         self._memo: dict = {}
         self.token_store = fn.token_store
-        self.request_slots: Optional[torch.Tensor] = None   # int32 [entries] on the device, where the step keeps them there (decode graphs)
+        self.request_slots: Optional[torch.Tensor] = None   # int32 [entries] on the device: the request slot of every entry
+        self.row_offsets: Optional[torch.Tensor] = None     # int32 [entries + 1] on the device: entry i owns the rows [i] .. [i+1]-1; None: one row each (decode graphs)
         self.want_slots: Optional[torch.Tensor] = None      # int32 [wanted rows] on the device: the request slot behind every wanted row
 
     @property
@@ -268,7 +269,9 @@ class StepFunction:
         width = cache.step_width(slots, n_tokens)
         # one pinned block, laid out in place, and one copy that the host does not wait for:
         # ids, positions, request of every token, wanted rows and their requests' slots, block tables (int32); cache slots (int64)
-        n32 = 3 * T + 2 * len(want) + G * n * width
+        # ... and, for parts that keep state per request, the requests' slots and where each one's rows begin
+        at_requests = 3 * T + 2 * len(want) + G * n * width
+        n32 = at_requests + 2 * n + 1
         n32 += n32 % 2
         nbytes = 4 * n32 + 8 * G * T
         host = self._eager_host(nbytes)
@@ -279,6 +282,9 @@ class StepFunction:
                              h32[at_tables:at_tables + G * n * width].reshape(G, n, width), h64.reshape(G, T))
         h32[:T] = ids
         spans = self._spans(entries, slots, n_tokens, pos0)
+        h32[at_requests:at_requests + n] = slots
+        h32[at_requests + n] = 0
+        np.cumsum(n_tokens, out=h32[at_requests + n + 1:at_requests + 2 * n + 1])
         if want:
             h32[at_rows:at_rows + len(want)] = [spans[i].row0 + w for i, w in want]
             h32[at_rows + len(want):at_tables] = [slots[i] for i, _ in want]      # the requests' places in the token store
@@ -292,6 +298,7 @@ class StepFunction:
         tables_d, slots_d = d32[at_tables:at_tables + G * n * width].view(G, n, width), d64.view(G, T)
         ctx._tables = [tables_d[g] for g in range(G)]
         ctx._slots = [slots_d[g] for g in range(G)]
+        ctx.request_slots, ctx.row_offsets = d32[at_requests:at_requests + n], d32[at_requests + n:at_requests + 2 * n + 1]
         rows = d32[at_rows:at_rows + len(want)] if want else None
         ctx.want_slots = d32[at_rows + len(want):at_tables] if want else None
         return ctx, ids_d, rows

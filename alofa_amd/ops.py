@@ -885,3 +885,210 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: torch.Tensor, u
     _store_operands(store, store_index, n)
     _call("alofa_sample", _ptr(out), _ptr(logits), _L(_rows("logits", logits)), _I(n), _I(logits.shape[1]), _ptr(temperature), _ptr(uniform),
           _ptr(store), _ptr(store_index), _stream())
+
+
+# ------------------------------------------------- layer norm, head norm, activations, sums over depth and branches
+
+def layernorm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: torch.Tensor, eps: float, exact: bool,
+              rows: Optional[torch.Tensor] = None, out_scale: float = 1.0) -> None:
+    """out[r] = (x[r'] - mean) / sqrt(var + eps) * w + b (times ``out_scale``), r' = rows[r] if given else r; var is the
+    mean of the squared deviations. ``out`` may be ``x`` itself."""
+    _gpu("out", out, None, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 1), _gpu("b", b, torch.float32, 1)
+    _contig("out", out), _contig("x", x), _contig("w", w), _contig("b", b)
+    n, h = out.shape
+    if x.shape[1] != h or w.shape[0] != h or b.shape[0] != h:
+        raise AlofaError("shape_mismatch", "norm width does not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)} b={tuple(b.shape)}")
+    if rows is not None:
+        _gpu("rows", rows, torch.int32, 1), _contig("rows", rows)
+        if rows.shape[0] != n:
+            raise AlofaError("shape_mismatch", "one row index per output row", f"rows={tuple(rows.shape)} out={tuple(out.shape)}")
+        if out.data_ptr() == x.data_ptr():
+            raise AlofaError("invalid_argument", "a norm of gathered rows cannot write over its input")
+    elif x.shape[0] != n:
+        raise AlofaError("shape_mismatch", "norm row count does not fit", f"out={tuple(out.shape)} x={tuple(x.shape)}")
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
+    _call("alofa_layernorm", _ptr(out), _I(dtype_code(out)), _ptr(x), _ptr(w), _ptr(b), _ptr(rows), _I(n), _I(h), _F(eps), _F(out_scale),
+          _I(int(exact)), _stream())
+
+
+def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], heads: int, dv: int,
+                  eps: float, exact: bool, out_scale: float = 1.0) -> None:
+    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * silu(gate[t, h, :]); ``o`` float32
+    [T, heads * dv] contiguous, ``gate`` and ``out`` rows of heads * dv in the activation dtype (row strides allowed),
+    ``weight`` float32 [heads * dv] or None."""
+    _gpu("out", out, None, 2), _gpu("o", o, torch.float32, 2), _gpu("gate", gate, out.dtype, 2), _contig("o", o)
+    T = o.shape[0]
+    if o.shape[1] != heads * dv or tuple(out.shape) != (T, heads * dv) or tuple(gate.shape) != (T, heads * dv):
+        raise AlofaError("shape_mismatch", "head norm operands do not fit", f"out={tuple(out.shape)} o={tuple(o.shape)} gate={tuple(gate.shape)} heads={heads} dv={dv}")
+    if weight is not None:
+        _gpu("weight", weight, torch.float32, 1), _contig("weight", weight)
+        if weight.shape[0] != heads * dv:
+            raise AlofaError("shape_mismatch", "one weight per head and channel", f"weight={tuple(weight.shape)} heads={heads} dv={dv}")
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
+    _call("alofa_headnorm_gate", _ptr(out), _L(_rows("out", out)), _ptr(o), _ptr(gate), _L(_rows("gate", gate)), _I(dtype_code(out)), _ptr(weight),
+          _I(T), _I(heads), _I(dv), _F(eps), _F(out_scale), _I(int(exact)), _stream())
+
+
+XIELU, TANH = 0, 1
+
+
+def activation(out: torch.Tensor, x: torch.Tensor, kind: int, a: float = 0.0, b: float = 0.0, exact: bool = False) -> None:
+    """out = act(x) element by element on rows ([T, n], row strides allowed; out may be x). ``XIELU`` with a = softplus(p),
+    b = 1/2 + softplus(q): z > 0: a z^2 + z/2, else b (exp(z) - 1 - z) + z/2. ``TANH``."""
+    _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2)
+    if out.shape != x.shape or kind not in (XIELU, TANH):
+        raise AlofaError("shape_mismatch", "activation operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} kind={kind}")
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
+    _call("alofa_activation", _ptr(out), _L(_rows("out", out)), _ptr(x), _L(_rows("x", x)), _I(dtype_code(out)), _L(x.shape[0]), _I(x.shape[1]),
+          _I(kind), _F(a), _F(b), _I(int(exact)), _stream())
+
+
+def depth_average(x: torch.Tensor, stack: torch.Tensor, weights: Optional[torch.Tensor], n: int, exact: bool = False) -> None:
+    """stack[n - 1] = x, then x = sum_{j < n} weights[j] * stack[j] (j ascending); without weights only the copy.
+    ``stack`` float32 [levels, *x.shape] contiguous."""
+    _gpu("x", x, torch.float32), _gpu("stack", stack, torch.float32), _contig("x", x), _contig("stack", stack)
+    if tuple(stack.shape[1:]) != tuple(x.shape) or not 1 <= n <= stack.shape[0]:
+        raise AlofaError("shape_mismatch", "the stack of levels does not fit", f"x={tuple(x.shape)} stack={tuple(stack.shape)} n={n}")
+    if weights is not None:
+        _gpu("weights", weights, torch.float32, 1), _contig("weights", weights)
+        if weights.shape[0] != n:
+            raise AlofaError("shape_mismatch", "one weight per level", f"weights={tuple(weights.shape)} n={n}")
+    _call("alofa_depth_average", _ptr(x), _ptr(stack), _L(x.numel()), _ptr(weights), _I(n), _L(x.numel()), _I(int(exact)), _stream())
+
+
+def add_scaled(residual: torch.Tensor, x: torch.Tensor, a: float, y: Optional[torch.Tensor] = None, b: float = 0.0, exact: bool = False) -> None:
+    """residual += a * x (+ b * y), all float32 of one shape."""
+    _gpu("residual", residual, torch.float32), _gpu("x", x, torch.float32), _contig("residual", residual), _contig("x", x)
+    if y is not None:
+        _gpu("y", y, torch.float32), _contig("y", y)
+    if x.shape != residual.shape or (y is not None and y.shape != residual.shape):
+        raise AlofaError("shape_mismatch", "the branches must have the residual stream's shape", f"residual={tuple(residual.shape)} x={tuple(x.shape)}")
+    _call("alofa_add_scaled", _ptr(residual), _ptr(x), _F(a), _ptr(y), _F(b), _L(residual.numel()), _I(int(exact)), _stream())
+
+
+def scale_(x: torch.Tensor, s: float) -> None:
+    """x *= s (float32, contiguous)."""
+    _gpu("x", x, torch.float32), _contig("x", x)
+    _call("alofa_scale", _ptr(x), _F(s), _L(x.numel()), _stream())
+
+
+# ------------------------------------------------------------- state of fixed size per request: rows, convolution, recurrence
+
+class RowsOfRequests:
+    """How a step's rows belong to requests, as the kernels of stateful parts read it from the device: ``slots`` int32
+    [R] (the state slot of request r of the step), ``offsets`` int32 [R + 1] (request r owns rows offsets[r] ..
+    offsets[r+1] - 1) or None when every request brings one row, ``req_of_row`` int32 [T] or None likewise."""
+
+    def __init__(self, slots: torch.Tensor, offsets: Optional[torch.Tensor], req_of_row: Optional[torch.Tensor], requests: int, rows: int, n_slots: int):
+        _gpu("slots", slots, torch.int32, 1), _contig("slots", slots)
+        if slots.shape[0] != requests or requests > rows:
+            raise AlofaError("shape_mismatch", "one state slot per request of the step", f"slots={tuple(slots.shape)} requests={requests} rows={rows}")
+        if offsets is None:
+            if requests != rows or req_of_row is not None:
+                raise AlofaError("shape_mismatch", "without offsets every request brings one row", f"requests={requests} rows={rows}")
+        else:
+            _gpu("offsets", offsets, torch.int32, 1), _contig("offsets", offsets), _gpu("req_of_row", req_of_row, torch.int32, 1), _contig("req_of_row", req_of_row)
+            if offsets.shape[0] != requests + 1 or req_of_row.shape[0] != rows:
+                raise AlofaError("shape_mismatch", "offsets hold one more than the requests, and every row names its request",
+                                 f"offsets={tuple(offsets.shape)} req_of_row={tuple(req_of_row.shape)} requests={requests} rows={rows}")
+        self.slots, self.offsets, self.req_of_row, self.requests, self.rows, self.n_slots = slots, offsets, req_of_row, requests, rows, n_slots
+
+    def fits(self, name: str, state: torch.Tensor) -> None:
+        if state.shape[0] < self.n_slots:
+            raise AlofaError("shape_mismatch", "the state has fewer slots than the step's requests may name", f"operand={name} state={tuple(state.shape)} slots={self.n_slots}")
+
+
+CONV_MAX_TAPS = 9
+
+
+def short_conv(out: torch.Tensor, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests, exact: bool = False) -> None:
+    """out[t] = h[t] + sum_j w[:, j] * h[t - taps + 1 + j] per channel, within each request; the rows before a request's
+    first row of this step come from ``state`` [slots, taps - 1, width] (h's dtype; the newest last), which is not
+    written (``keep_last_rows`` does that afterwards). ``w`` float32 [width, taps]."""
+    _gpu("out", out, None, 2), _gpu("h", h, None, 2), _gpu("w", w, torch.float32, 2), _gpu("state", state, h.dtype, 3)
+    _contig("out", out), _contig("h", h), _contig("w", w), _contig("state", state)
+    T, width = h.shape
+    taps = w.shape[1]
+    if tuple(out.shape) != (T, width) or w.shape[0] != width or tuple(state.shape[1:]) != (taps - 1, width) or T != rows.rows or not 1 <= taps <= CONV_MAX_TAPS:
+        raise AlofaError("shape_mismatch", "convolution operands do not fit", f"out={tuple(out.shape)} h={tuple(h.shape)} w={tuple(w.shape)} state={tuple(state.shape)} rows={rows.rows}")
+    rows.fits("state", state)
+    if exact and (out.dtype is not torch.float32 or h.dtype is not torch.float32):
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout")
+    _call("alofa_short_conv", _ptr(out), _I(dtype_code(out)), _ptr(h), _I(dtype_code(h)), _ptr(w), _ptr(state), _ptr(rows.slots), _ptr(rows.offsets),
+          _ptr(rows.req_of_row), _I(T), _I(width), _I(taps), _I(int(exact)), _stream())
+
+
+def keep_last_rows(state: torch.Tensor, h: torch.Tensor, rows: RowsOfRequests) -> None:
+    """state[slot] [keep, width] = the last ``keep`` rows its request has seen once this step's rows ``h`` are in (older
+    ones from the state itself where the step brought fewer)."""
+    _gpu("state", state, h.dtype, 3), _gpu("h", h, None, 2), _contig("state", state), _contig("h", h)
+    if state.shape[2] != h.shape[1] or h.shape[0] != rows.rows or state.shape[1] > CONV_MAX_TAPS - 1:
+        raise AlofaError("shape_mismatch", "the kept rows do not fit", f"state={tuple(state.shape)} h={tuple(h.shape)} rows={rows.rows}")
+    rows.fits("state", state)
+    _call("alofa_keep_last_rows", _ptr(state), _ptr(h), _I(dtype_code(h)), _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(h.shape[1]),
+          _I(state.shape[1]), _stream())
+
+
+def shift_mix(out: torch.Tensor, x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests) -> None:
+    """out[s, t] = x[t] + (x[t - 1] - x[t]) * mu[s], the row before a request's first row of this step taken from
+    ``state`` [slots, 1, width] (x's dtype; not written). ``mu`` float32 [n, width]; out [n, T, width] in x's dtype."""
+    _gpu("out", out, x.dtype, 3), _gpu("x", x, None, 2), _gpu("mu", mu, torch.float32, 2), _gpu("state", state, x.dtype, 3)
+    _contig("out", out), _contig("x", x), _contig("mu", mu), _contig("state", state)
+    T, width = x.shape
+    if tuple(out.shape) != (mu.shape[0], T, width) or mu.shape[1] != width or tuple(state.shape[1:]) != (1, width) or T != rows.rows:
+        raise AlofaError("shape_mismatch", "token mix operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} mu={tuple(mu.shape)} state={tuple(state.shape)}")
+    rows.fits("state", state)
+    _call("alofa_shift_mix", _ptr(out), _ptr(x), _I(dtype_code(x)), _ptr(mu), _ptr(state), _ptr(rows.slots), _ptr(rows.offsets), _ptr(rows.req_of_row),
+          _I(T), _I(width), _I(mu.shape[0]), _stream())
+
+
+DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP = 0, 1, 2
+RECURRENCE_MAX_KEYS = 512
+
+
+def recurrence_chunk(dk: int) -> int:
+    """Rows that the recurrence kernel stages in LDS at a time: sixteen, or as many as 64 KB hold for long keys."""
+    chunk = 16
+    while chunk > 1 and _recurrence_lds(dk, chunk) > 64 * 1024:
+        chunk //= 2
+    return chunk
+
+
+def _recurrence_lds(dk: int, chunk: int) -> int:
+    return int(load().alofa_linear_recurrence_lds_bytes(_I(dk), _I(chunk)))
+
+
+def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests,
+                      heads: int, dk: int, dv: int, decay_kind: int, decay: torch.Tensor, tau: float = 1.0, bonus: Optional[torch.Tensor] = None,
+                      q_scale: float = 1.0, k_scale: float = 1.0, before_update: bool = False) -> None:
+    """Per request (in its rows' order) and head: S = diag(w_t) S + k_t v_t^T and out_t = S^T q_t, or with
+    ``before_update`` out_t = (S + diag(bonus) k_t v_t^T)^T q_t first and the update after it. S float32
+    [slots, heads, dk, dv] is read and left in ``state``. q, k [T, heads * dk] and v [T, heads * dv] are rows in one
+    dtype (row strides allowed); ``out`` float32 [T, heads * dv]. The decay w_t: ``DECAY_PER_HEAD`` with ``decay``
+    float32 [heads]; ``DECAY_SIGMOID_ROOT`` sigmoid(z)^(1/tau) or ``DECAY_EXP_NEG_EXP`` exp(-exp(z)) with ``decay`` = z
+    float32 [T, heads * dk] rows."""
+    _gpu("out", out, torch.float32, 2), _contig("out", out), _gpu("q", q, None, 2), _gpu("k", k, q.dtype, 2), _gpu("v", v, q.dtype, 2)
+    _gpu("state", state, torch.float32, 4), _contig("state", state)
+    T = q.shape[0]
+    if (tuple(q.shape) != (T, heads * dk) or tuple(k.shape) != (T, heads * dk) or tuple(v.shape) != (T, heads * dv) or tuple(out.shape) != (T, heads * dv)
+            or tuple(state.shape[1:]) != (heads, dk, dv) or T != rows.rows or not 0 < dk <= RECURRENCE_MAX_KEYS):
+        raise AlofaError("shape_mismatch", "recurrence operands do not fit", f"q={tuple(q.shape)} k={tuple(k.shape)} v={tuple(v.shape)} out={tuple(out.shape)} "
+                         f"state={tuple(state.shape)} heads={heads} dk={dk} dv={dv} rows={rows.rows}")
+    rows.fits("state", state)
+    per_head = decay_kind == DECAY_PER_HEAD
+    _gpu("decay", decay, torch.float32, 1 if per_head else 2)
+    if per_head:
+        _contig("decay", decay)
+    if (tuple(decay.shape) != (heads,)) if per_head else (tuple(decay.shape) != (T, heads * dk)) or decay_kind not in (DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP):
+        raise AlofaError("shape_mismatch", "the decay does not fit its kind", f"decay={tuple(decay.shape)} kind={decay_kind} heads={heads} dk={dk}")
+    if bonus is not None:
+        _gpu("bonus", bonus, torch.float32, 2), _contig("bonus", bonus)
+        if tuple(bonus.shape) != (heads, dk) or not before_update:
+            raise AlofaError("shape_mismatch", "the bonus is [heads, dk] and goes with the read-out before the update", f"bonus={tuple(bonus.shape)}")
+    _call("alofa_linear_recurrence", _ptr(out), _ptr(q), _L(_rows("q", q)), _ptr(k), _L(_rows("k", k)), _ptr(v), _L(_rows("v", v)), _I(dtype_code(q)),
+          _ptr(None if per_head else decay), _L(0 if per_head else _rows("decay", decay)), _ptr(decay if per_head else None), _ptr(bonus), _ptr(state),
+          _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(heads), _I(dk), _I(dv), _I(decay_kind), _F(tau), _F(q_scale), _F(k_scale),
+          _I(int(before_update)), _I(recurrence_chunk(dk)), _stream())

@@ -17,7 +17,7 @@ import torch
 from .. import ops
 from ..errors import AlofaError
 from ..weights.loader import TensorRule
-from .base import CacheNeed, Mixer, build_part, register_part
+from .base import CacheNeed, Mixer, build_part, part_class, register_part
 
 
 SHORT = ops.DECODE_MAX_Q     # rows of one request up to which they are served as single tokens
@@ -57,28 +57,67 @@ class RowPlan:
         return self._tiles[key]
 
 
+NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
+         "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias"}
+
+
+def _padded_heads(t: torch.Tensor, heads: int, size: int, to: int, order=None) -> torch.Tensor:
+    """Rows of ``t`` are ``heads`` heads of ``size`` channels: every head widened to ``to`` channels by zero rows, then
+    its channels put in ``order`` (indices into the widened head)."""
+    if size == to and order is None:
+        return t
+    rest = tuple(t.shape[1:])
+    t = t.reshape(heads, size, *rest)
+    if to > size:
+        t = torch.cat([t, torch.zeros((heads, to - size, *rest), dtype=t.dtype)], dim=1)
+    if order is not None:
+        t = t[:, torch.tensor(order, dtype=torch.long)]
+    return t.reshape(heads * to, *rest).contiguous()
+
+
 class GQAAttention(Mixer):
     """params: prefix, hidden, heads, kv_heads, head_dim, qkv_bias, out_bias,
-    window (None or a count of keys), position (PartSpec)."""
+    window (None or a count of keys), position (PartSpec); optional: v_head_dim (the size of a value head, default
+    head_dim), scale (what scores are multiplied by, default 1/sqrt(head_dim)), names (tensor names after the prefix
+    for q, k, v, o and their biases, default the *_proj ones), init (the rule random weights are drawn by).
+
+    The kernels know one head size d. Where query/key and value heads differ in size, or the size is none the
+    prefill kernel is built for, every head is widened to a common d with zero rows in its projection (zero columns
+    in the output matrix): products with zeros change nothing."""
     capturable = True   # native kernels on the current stream only: a decode step may be graph-captured
 
     @classmethod
     def tensors(cls, spec):
         p = spec.params
-        pre, h, qd, kvd = p["prefix"], p["hidden"], p["heads"] * p["head_dim"], p["kv_heads"] * p["head_dim"]
-        out = {pre + "q_proj.weight": TensorRule((qd, h)), pre + "k_proj.weight": TensorRule((kvd, h)),
-               pre + "v_proj.weight": TensorRule((kvd, h)), pre + "o_proj.weight": TensorRule((h, qd))}
+        names, init = {**NAMES, **p.get("names", {})}, p.get("init", "matrix")
+        dv = p.get("v_head_dim") or p["head_dim"]
+        pre, h, qd, kd, vd, od = p["prefix"], p["hidden"], p["heads"] * p["head_dim"], p["kv_heads"] * p["head_dim"], p["kv_heads"] * dv, p["heads"] * dv
+        out = {pre + names["q"]: TensorRule((qd, h), init), pre + names["k"]: TensorRule((kd, h), init),
+               pre + names["v"]: TensorRule((vd, h), init), pre + names["o"]: TensorRule((h, od), init)}
         if p.get("qkv_bias", False):
-            out.update({pre + "q_proj.bias": TensorRule((qd,), "bias"), pre + "k_proj.bias": TensorRule((kvd,), "bias"),
-                        pre + "v_proj.bias": TensorRule((kvd,), "bias")})
+            out.update({pre + names["q_bias"]: TensorRule((qd,), "bias"), pre + names["k_bias"]: TensorRule((kd,), "bias"),
+                        pre + names["v_bias"]: TensorRule((vd,), "bias")})
         if p.get("out_bias", False):
-            out[pre + "o_proj.bias"] = TensorRule((h,), "bias")
+            out[pre + names["o_bias"]] = TensorRule((h,), "bias")
         return out
+
+    @staticmethod
+    def common_head_size(qk: int, v: int) -> int:
+        """The one head size the kernels run with: the larger of the two; when they differ, or the size is odd, the
+        next size the prefill kernel is built for, if there is one."""
+        d = max(qk, v)
+        d += d % 2
+        if qk != v or d != qk:
+            d = next((n for n in ops.PREFILL_HEAD_DIMS if n >= d), d)
+        return d
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p = spec.params
-        self.hidden, self.heads, self.kv_heads, self.d = int(p["hidden"]), int(p["heads"]), int(p["kv_heads"]), int(p["head_dim"])
+        self.hidden, self.heads, self.kv_heads = int(p["hidden"]), int(p["heads"]), int(p["kv_heads"])
+        self.qk_dim = int(p["head_dim"])
+        self.v_dim = int(p.get("v_head_dim") or self.qk_dim)
+        self.d = self.common_head_size(self.qk_dim, self.v_dim)
         self.window = p.get("window")
         if self.kv_heads <= 0 or self.heads % self.kv_heads:
             raise AlofaError("unsupported", "kv_heads must be positive and divide heads", f"heads={self.heads} kv_heads={self.kv_heads}")
@@ -88,18 +127,26 @@ class GQAAttention(Mixer):
         self.mfma_heads = self.d % 16 == 0
         if self.window is not None and self.window <= 0:
             raise AlofaError("invalid_argument", "an attention window must be positive", f"window={self.window}")
-        pre = p["prefix"]
-        mats = [weights[pre + n + "_proj.weight"] for n in ("q", "k", "v")]
+        pre, names = p["prefix"], {**NAMES, **p.get("names", {})}
+        position = p["position"]
+        if self.d != self.qk_dim:
+            position = part_class("position", position.kind).for_head(position, self.d)
+        self.position = build_part("position", position, weights, rt)
+        order = self.position.channel_order()      # (the order of a head's channels in which the encoding's pairs lie as the kernels pair them)
+        sizes = {"q": (self.heads, self.qk_dim, order), "k": (self.kv_heads, self.qk_dim, order), "v": (self.kv_heads, self.v_dim, None)}
+        mats = [_padded_heads(weights[pre + names[n]], *sizes[n][:2], self.d, sizes[n][2]) for n in ("q", "k", "v")]
         if len({m.dtype for m in mats}) > 1:
             mats = [m.float() for m in mats]
         self.w_qkv = rt.matrix(torch.cat(mats, dim=0))
-        self.b_qkv = (rt.vector(torch.cat([weights[pre + n + "_proj.bias"].float() for n in ("q", "k", "v")]))
+        self.b_qkv = (rt.vector(torch.cat([_padded_heads(weights[pre + names[n + "_bias"]].float(), *sizes[n][:2], self.d, sizes[n][2]) for n in ("q", "k", "v")]))
                       if p.get("qkv_bias", False) else None)
-        self.w_o = rt.matrix(weights[pre + "o_proj.weight"])
-        self.b_o = rt.vector(weights[pre + "o_proj.bias"]) if p.get("out_bias", False) else None
-        self.position = build_part("position", p["position"], weights, rt)
-        # float32 1 / sqrt(float32 d), as the reference forms it (scalar.mojo:421)
-        self.scale = float(np.float32(1.0) / np.sqrt(np.float32(self.d)))
+        w_o = weights[pre + names["o"]]
+        if self.d != self.v_dim:      # zero columns where the value heads were widened
+            w_o = _padded_heads(w_o.t(), self.heads, self.v_dim, self.d).t()
+        self.w_o = rt.matrix(w_o)
+        self.b_o = rt.vector(weights[pre + names["o_bias"]]) if p.get("out_bias", False) else None
+        # float32 1 / sqrt(float32 d), as the reference forms it (scalar.mojo:421), unless the configuration gives the factor
+        self.scale = float(p["scale"]) if p.get("scale") is not None else float(np.float32(1.0) / np.sqrt(np.float32(self.qk_dim)))
         self.qkv_width = (self.heads + 2 * self.kv_heads) * self.d
         # an encoding applied by other code (``apply``) is captured only if it says that it may be: native kernels or
         # library calls on the current stream that allocate nothing and record no memset
@@ -119,7 +166,8 @@ class GQAAttention(Mixer):
     def gives_normed(self):
         return self.b_o is None
 
-    def forward(self, ctx, entry, x, residual, norm=None, then=None):
+    def forward(self, ctx, entry, x, residual, norm=None, then=None, out=None):
+        """``out`` (float32, the residual's shape): the mix is stored there instead of being added to the residual."""
         T = residual.shape[0]
         exact = self.rt.exact
         qkv = ctx.scratch("qkv", (T, self.qkv_width), self.rt.dtype)
@@ -163,7 +211,9 @@ class GQAAttention(Mixer):
                 one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
                 ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
                                      ctx.max_context, partial, rows=plan.short_rows, rope=(cos, sin, kv.slots) if fused else None)
-        if self.b_o is not None:
+        if out is not None:
+            ops.gemm(out, attn, self.w_o, self.b_o, exact=exact)
+        elif self.b_o is not None:
             proj = ctx.scratch("attn_proj", (T, self.hidden), torch.float32)
             ops.gemm(proj, attn, self.w_o, self.b_o, exact=exact)
             residual.add_(proj)

@@ -7,6 +7,7 @@ dtype, ``residual`` the float32 residual stream):
 
   norm          forward(out[n,h], x[T,h] f32, rows=None)         out = norm(x[rows])
   position      table(n_positions) -> (cos, sin) f32 [n, d/2], or apply(ctx, q, k)
+  conv          forward(ctx, where, out[T,h], x[T,h] f32)         out = x + conv over time(x), per request; state_need()
   mixer         forward(ctx, where, x, residual)                  residual += mix(x)
                 cache_need() -> CacheNeed | None, state_need() -> StateNeed | None,
                 prepare(n_positions), capturable
@@ -27,7 +28,7 @@ import torch
 from ..config.base import PartSpec
 from ..errors import AlofaError
 
-FAMILIES = ("embedding", "norm", "position", "mixer", "feed_forward", "block", "head")
+FAMILIES = ("embedding", "norm", "position", "conv", "mixer", "feed_forward", "block", "head")
 _REGISTRY = {f: {} for f in FAMILIES}
 
 
@@ -154,7 +155,34 @@ class Mixer(Part):
     # ``norm`` of the residual's new rows in ``rows`` (the activation dtype), however it gets there.
     gives_normed = False
 
+    def stateful_parts(self) -> list:
+        """The parts that keep a cache or state, in a fixed order: the mixer itself, or, for a mixer made of several,
+        theirs one after the other. A mixer called with ``where`` = (entry, k) reaches the j-th of them as (entry, k + j)."""
+        return [self]
+
     def forward(self, ctx, where, x: torch.Tensor, residual: torch.Tensor) -> None:
+        """``residual += mix(x)``. Mixers that may stand beside others in one layer also take ``out=`` (float32, the
+        residual's shape): the mix is stored there and the residual left alone."""
+        raise NotImplementedError
+
+
+class TimeConv(Part):
+    """A filter over time on the rows a sub-layer reads, within each request. What it has to remember of the rows
+    before a step is state of fixed size: a block lists it among its ``mixers()`` so that it gets a place
+    (``where``) to keep it."""
+    family = "conv"
+    capturable = False
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def prepare(self, n_positions: int) -> None:
+        pass
+
+    def forward(self, ctx, where, out: torch.Tensor, x: torch.Tensor) -> None:
         raise NotImplementedError
 
 
@@ -241,6 +269,16 @@ class PositionEncoding(Part):
         """(cos, sin) float32 [n_positions, d/2] on the device for encodings that
         rotate pairs (j, j + d/2) by a position-dependent angle; None otherwise."""
         return None
+
+    def channel_order(self):
+        """None, or the order of a head's channels (a list of head_dim indices into the stored order) in which the
+        encoding's pairs lie as the table has them, (j, j + head_dim/2): queries and keys are projected in that order."""
+        return None
+
+    @classmethod
+    def for_head(cls, spec: PartSpec, head_dim: int) -> PartSpec:
+        """The same encoding for a head widened to ``head_dim`` channels, the added ones passing unchanged."""
+        return PartSpec(spec.kind, {**spec.params, "head_dim": int(head_dim)})
 
     def apply(self, ctx, q: torch.Tensor, k: torch.Tensor) -> None:
         """In-place encoding of q [T, heads, d] and k [T, kv_heads, d] views, for

@@ -3,10 +3,17 @@
 prenorm: a = hidden; a += mixer(norm0(a)); a += feed_forward(norm1(a)) — two
 norms before their sub-layers, two residual sums in float32
 (src/alofa/model/arch/qwen.mojo:1418-1510). It reads the layer's parts
-``mixer``, ``feed_forward`` and ``norms`` (two)."""
+``mixer``, ``feed_forward`` and ``norms`` (two).
+
+filtered_prenorm: the same with a filter over time in front of every sub-layer, an optional feed-forward, and an
+optional weighted average over the outputs of all layers so far."""
 from __future__ import annotations
 
+import torch
+
+from .. import ops
 from ..errors import AlofaError
+from ..weights.loader import TensorRule
 from .base import Block, build_part, register_part, tensors_of
 
 
@@ -69,4 +76,79 @@ class PreNormBlock(Block):
         return given
 
 
+class FilteredPreNormBlock(Block):
+    """a += mixer(conv0(norm0(a))), then, where the layer has a feed-forward, a += feed_forward(conv1(norm1(a))): the
+    rows every sub-layer reads pass a filter over time first (a part of the "conv" family that keeps its own state).
+    Then, with ``depth_average`` (a tensor of as many weights as there are layer outputs so far, the embedding's
+    counted), what goes on is the weighted sum of the outputs of all layers up to this one, each taken before its
+    own averaging; the outputs live in a stack that the step keeps.
+
+    It reads the layer's parts ``mixer``, ``norms`` and ``convs`` (one per sub-layer; a conv may be None) and
+    ``feed_forward`` (may be None). params: depth_average (tensor name or None), level (this layer's place in
+    the stack: it has level + 1 weights), levels (the stack's height), hidden."""
+
+    @classmethod
+    def layer_tensors(cls, layer) -> dict:
+        out = {}
+        for n in layer.part("norms"):
+            out.update(tensors_of("norm", n))
+        for c in layer.part("convs"):
+            if c is not None:
+                out.update(tensors_of("conv", c))
+        out.update(tensors_of("mixer", layer.part("mixer")))
+        if layer.part("feed_forward") is not None:
+            out.update(tensors_of("feed_forward", layer.part("feed_forward")))
+        if layer.block.get("depth_average") is not None:
+            out[layer.block.params["depth_average"]] = TensorRule((layer.block.params["level"] + 1,), "average")
+        return out
+
+    def __init__(self, layer, weights, rt):
+        super().__init__(layer, weights, rt)
+        p = layer.block.params
+        ff = layer.part("feed_forward")
+        subs = 1 if ff is None else 2
+        norms, convs = layer.part("norms"), layer.part("convs")
+        if len(norms) != subs or len(convs) != subs:
+            raise AlofaError("invalid_argument", "one norm and one filter (or None) per sub-layer", f"prefix={layer.prefix} sub-layers={subs} norms={len(norms)} convs={len(convs)}")
+        self.norms = [build_part("norm", n, weights, rt) for n in norms]
+        self.convs = [build_part("conv", c, weights, rt) if c is not None else None for c in convs]
+        self.mixer = build_part("mixer", layer.part("mixer"), weights, rt)
+        self.feed_forward = build_part("feed_forward", ff, weights, rt) if ff is not None else None
+        self.level, self.levels = int(p.get("level", 0)), int(p.get("levels", 0))
+        self.depth_weights = rt.vector(weights[p["depth_average"]]) if p.get("depth_average") is not None else None
+        if self.depth_weights is not None and not 1 <= self.level < self.levels:
+            raise AlofaError("invalid_argument", "a layer's level lies above the embedding's and within the stack", f"level={self.level} levels={self.levels}")
+        self.parts = [p for p in (*self.norms, *self.convs, self.mixer, self.feed_forward) if p is not None]
+        # the parts that keep a cache or state: the mixer's, then the filters
+        self._stateful = [*self.mixer.stateful_parts(), *(c for c in self.convs if c is not None)]
+
+    def mixers(self):
+        return self._stateful
+
+    def _read(self, ctx, entry, sub, hidden):
+        """What sub-layer ``sub`` reads: its norm of the stream, filtered over time, in the activation dtype."""
+        rows = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
+        conv = self.convs[sub]
+        if conv is None:
+            self.norms[sub].forward(rows, hidden)
+            return rows
+        wide = ctx.scratch("normed_f32", tuple(hidden.shape), torch.float32)
+        self.norms[sub].forward(wide, hidden)
+        conv.forward(ctx, (entry, self._stateful.index(conv)), rows, wide)
+        return rows
+
+    def forward(self, ctx, entry, hidden):
+        stack = None
+        if self.depth_weights is not None:
+            stack = ctx.scratch("depth_stack", (self.levels, *hidden.shape), torch.float32)
+            if self.level == 1:      # what the layers start from is the lowest level
+                ops.depth_average(hidden, stack, None, 1, self.rt.exact)
+        self.mixer.forward(ctx, (entry, 0), self._read(ctx, entry, 0, hidden), hidden)
+        if self.feed_forward is not None:
+            self.feed_forward.forward(ctx, self._read(ctx, entry, 1, hidden), hidden)
+        if stack is not None:
+            ops.depth_average(hidden, stack, self.depth_weights, self.level + 1, self.rt.exact)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "filtered_prenorm", FilteredPreNormBlock)

@@ -10,41 +10,49 @@ import torch
 from .. import ops
 from ..errors import AlofaError
 from ..weights.loader import TensorRule
-from .base import Part, register_part
+from .base import Part, build_part, register_part, tensors_of
 
 
 class TokenEmbedding(Part):
-    """params: name, vocab, width."""
+    """params: name, vocab, width; optional: norm (PartSpec of a norm applied to the looked-up rows), init."""
     family = "embedding"
 
     @classmethod
     def tensors(cls, spec):
-        return {spec.params["name"]: TensorRule((spec.params["vocab"], spec.params["width"]))}
+        out = {spec.params["name"]: TensorRule((spec.params["vocab"], spec.params["width"]), spec.params.get("init", "matrix"))}
+        if spec.params.get("norm") is not None:
+            out.update(tensors_of("norm", spec.params["norm"]))
+        return out
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         self.vocab, self.width = int(spec.params["vocab"]), int(spec.params["width"])
         self.table = rt.matrix(weights[spec.params["name"]])
+        self.norm = build_part("norm", spec.params["norm"], weights, rt) if spec.params.get("norm") is not None else None
 
     def forward(self, ctx, ids):
         hidden = ctx.scratch("hidden", (ids.shape[0], self.width), torch.float32)
         ops.embed_gather(hidden, self.table, ids, getattr(ctx, "token_store", None))
+        if self.norm is not None:      # (float32 rows, normed where they lie)
+            self.norm.forward(hidden, hidden)
         return hidden
 
 
 class LMHead(Part):
-    """params: name, tied_to (embedding tensor name or None), vocab, width."""
+    """params: name, tied_to (embedding tensor name or None), vocab, width; optional: scale (the logits are multiplied
+    by it), init."""
     family = "head"
 
     @classmethod
     def tensors(cls, spec):
         p = spec.params
-        return {p["name"]: TensorRule((p["vocab"], p["width"]), optional=p.get("tied_to") is not None)}
+        return {p["name"]: TensorRule((p["vocab"], p["width"]), p.get("init", "matrix"), optional=p.get("tied_to") is not None)}
 
     def __init__(self, spec, weights, rt, embedding=None):
         super().__init__(spec, weights, rt)
         p = spec.params
         self.vocab = int(p["vocab"])
+        self.scale = float(p.get("scale", 1.0))
         if p["name"] in weights:
             self.weight = rt.matrix(weights[p["name"]])
         elif p.get("tied_to") is not None and embedding is not None:
@@ -55,12 +63,14 @@ class LMHead(Part):
     def forward(self, ctx, y):
         logits = ctx.scratch("logits", (y.shape[0], self.vocab), torch.float32)
         ops.gemm(logits, y, self.weight, exact=self.rt.exact)
+        if self.scale != 1.0:
+            ops.scale_(logits, self.scale)
         return logits
 
     def greedy(self, ctx, y, out, store=None, store_index=None):
         """out[r] = the first index of row r's highest logit (and store[store_index[r]], when
         given), without the logits where the product can take the argmax with it."""
-        if not self.rt.exact and ops.can_gemm_argmax(y.shape[0], self.weight):
+        if not self.rt.exact and self.scale > 0 and ops.can_gemm_argmax(y.shape[0], self.weight):      # (a positive scale moves no maximum)
             ops.gemm_argmax(out, y, self.weight, store=store, store_index=store_index)
         else:
             ops.argmax(out, self.forward(ctx, y), store=store, store_index=store_index)

@@ -1,10 +1,18 @@
-"""Dense SwiGLU feed-forward: down(silu(gate(x)) * up(x)), no biases; silu is
+"""Dense feed-forwards.
+
+SwiGLU: down(silu(gate(x)) * up(x)), no biases; silu is
 x / (1 + exp(-x)) (src/alofa/kernels/cpu/scalar.mojo:219-231,
 src/alofa/engine/executor.mojo:806-837). Gate and up run as one kernel that
-applies the activation before anything is written."""
+applies the activation before anything is written.
+
+Two matrices with an activation between them: down(act(up(x))), no biases. The activation xIELU has two numbers
+p, q of its own per layer: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
 from __future__ import annotations
 
+import math
+
 from .. import ops
+from ..errors import AlofaError
 from ..weights.loader import TensorRule
 from .base import FeedForward, register_part
 
@@ -50,4 +58,38 @@ class SwiGLU(FeedForward):
         ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact, then_norm=then_norm)
 
 
+def _softplus(z: float) -> float:
+    return math.log1p(math.exp(-abs(z))) + max(z, 0.0)
+
+
+class DenseActivated(FeedForward):
+    """params: prefix, hidden, intermediate, activation ("xielu"), names (after the prefix: up, down, act)."""
+    capturable = True
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, i, names = p["prefix"], p["hidden"], p["intermediate"], p["names"]
+        return {pre + names["up"]: TensorRule((i, h), "fan_in"), pre + names["down"]: TensorRule((h, i), "fan_in"), pre + names["act"]: TensorRule((2,), "bias")}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        if p.get("activation", "xielu") != "xielu":
+            raise AlofaError("unsupported", "no such activation is built", f"activation={p['activation']}")
+        self.hidden, self.intermediate = int(p["hidden"]), int(p["intermediate"])
+        pre, names = p["prefix"], p["names"]
+        self.w_up, self.w_down = rt.matrix(weights[pre + names["up"]]), rt.matrix(weights[pre + names["down"]])
+        # the two numbers are fixed once the weights are: what the kernel needs of them is formed here, in float64
+        pq = weights[pre + names["act"]].double().tolist()
+        self.a, self.b = _softplus(pq[0]), 0.5 + _softplus(pq[1])
+
+    def forward(self, ctx, x, residual):
+        act = ctx.scratch("ff_act", (residual.shape[0], self.intermediate), self.rt.dtype)
+        ops.gemm(act, x, self.w_up, exact=self.rt.exact)
+        ops.activation(act, act, ops.XIELU, self.a, self.b, self.rt.exact)
+        ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
+
+
 register_part("feed_forward", "swiglu", SwiGLU)
+register_part("feed_forward", "dense_activated", DenseActivated)

@@ -12,17 +12,28 @@ import math
 import numpy as np
 import torch
 
+from ..config.base import PartSpec
 from ..errors import AlofaError
 from .base import PositionEncoding, register_part
 
 
 class Rotary(PositionEncoding):
-    """params: theta, head_dim, pairing ("half")."""
+    """params: theta, head_dim, pairing ("half"), dims (how many of a head's first channels are rotated, default all
+    of them: channel i < dims/2 is paired with i + dims/2, the angle is p * theta^(-2i/dims), the channels from
+    ``dims`` on pass unchanged).
+
+    The kernels pair channel j with j + head_dim/2. With dims < head_dim the table holds the angle zero for the pairs
+    beyond dims/2, and ``channel_order`` names the order of a head's channels in which the design's pairs lie that
+    way: whoever projects queries and keys puts their channels in that order (both alike, so their products do not
+    change)."""
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         self.theta = float(spec.params["theta"])
         self.head_dim = int(spec.params["head_dim"])
+        self.dims = int(spec.params.get("dims") or self.head_dim)
+        if self.dims <= 0 or self.dims % 2 or self.dims > self.head_dim:
+            raise AlofaError("unsupported", "rotated channels: an even count, at most the head's size", f"dims={self.dims} head_dim={self.head_dim}")
         if spec.params.get("pairing", "half") != "half":
             raise AlofaError("unsupported", "only the half-split pairing (j, j + d/2) is built", f"pairing={spec.params['pairing']}")
         if self.head_dim <= 0 or self.head_dim % 2:
@@ -30,18 +41,31 @@ class Rotary(PositionEncoding):
 
     def host_table(self, n_positions: int):
         half = self.head_dim // 2
-        inv = np.empty(half, dtype=np.float32)
-        for i in range(half):
-            inv[i] = np.float32(1.0) / np.float32(math.pow(self.theta, (2.0 * i) / self.head_dim))
+        inv = np.zeros(half, dtype=np.float32)      # (pairs beyond dims/2 keep the angle zero: they pass unchanged)
+        for i in range(self.dims // 2):
+            inv[i] = np.float32(1.0) / np.float32(math.pow(self.theta, (2.0 * i) / self.dims))
         ang = np.arange(n_positions, dtype=np.float32)[:, None] * inv[None, :]
         ang = ang.astype(np.float32).astype(np.float64)
         return np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+    def channel_order(self):
+        if self.dims == self.head_dim:
+            return None
+        r, rest = self.dims // 2, (self.head_dim - self.dims) // 2
+        return [*range(r), *range(self.dims, self.dims + rest), *range(r, self.dims), *range(self.dims + rest, self.head_dim)]
+
+    @classmethod
+    def for_head(cls, spec, head_dim: int):
+        p = dict(spec.params)
+        p["dims"] = int(p.get("dims") or p["head_dim"])
+        p["head_dim"] = int(head_dim)
+        return PartSpec(spec.kind, p)
 
     def table(self, n_positions: int):
         """One table per (theta, head size) serves every layer of the model (kept on the runtime).
         A table that has to grow is replaced; the old one is kept alive, since a captured graph
         may still read it (for positions it covers)."""
-        key = ("rotary", self.theta, self.head_dim)
+        key = ("rotary", self.theta, self.head_dim, self.dims)
         have = self.rt.shared.get(key)
         if have is None or have[0].shape[0] < n_positions:
             n = max(n_positions, 2 * have[0].shape[0] if have else 0)

@@ -1,0 +1,283 @@
+"""Mixers that keep a state of fixed size per request instead of keys: per head a matrix S [dk, dv] in float32 that
+every token decays and adds to, S_t = diag(w_t) S_(t-1) + k_t v_t^T, and reads out with its query. They differ in
+where the decay comes from and in the order of read-out and update; the recurrence itself is one kernel
+(``ops.linear_recurrence``), and so are the norm of every head's read-out with the gate (``ops.headnorm_gate``).
+
+retention       w = a constant per head; rotary positions on q and k; k scaled by dk^(-1/2); o_t = S_t^T q_t;
+                o / rms(o) per head, times silu(gate), output projection.
+gated_linear    w_t = sigmoid(z_t)^(1/tau) per key channel, z = W_a2 (W_a1 x) + b; q scaled by dk^(-1/2); o_t = S_t^T q_t;
+                RMS norm per head with a weight shared by the heads, times silu(gate), output projection.
+time_mix        RWKV-style: each of r, k, v, g, w reads its own mix of the token with the one before it,
+                x + (x' - x) mu_s; w_t = exp(-exp(W_w2 tanh(W_w1 mix_w) + w0)); o_t = (S_(t-1) + diag(u) k_t v_t^T)^T r_t,
+                then the update; o / rms(o) per head, times a weight per channel, times silu(g), output projection.
+
+Projections and gates run in the activation dtype; decays, the state, the read-out and the head norms in float32.
+Every one of them takes ``out=`` (see ``Mixer.forward``)."""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from ..config.base import PartSpec
+from ..errors import AlofaError
+from ..weights.loader import TensorRule
+from .base import Mixer, StateNeed, TimeConv, build_part, register_part
+from .rows import rows_of_requests
+
+
+def _stacked(rt, mats: list) -> torch.Tensor:
+    if len({m.dtype for m in mats}) > 1:
+        mats = [m.float() for m in mats]
+    return rt.matrix(torch.cat(mats, dim=0))
+
+
+def _heads_in_order(t: torch.Tensor, heads: int, size: int, order) -> torch.Tensor:
+    if order is None:
+        return t
+    rest = tuple(t.shape[1:])
+    return t.reshape(heads, size, *rest)[:, torch.tensor(order, dtype=torch.long)].reshape(heads * size, *rest).contiguous()
+
+
+class RecurrentMixer(Mixer):
+    """What the three kinds share: sizes, the state, the way out (head norm, gate, output projection)."""
+    capturable = True   # native kernels on the current stream only: a decode step may be graph-captured
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.heads, self.dk = int(p["hidden"]), int(p["heads"]), int(p["key_dim"])
+        self.dv = int(p.get("value_dim") or self.dk)
+        self.eps = float(p["eps"])
+        if self.heads <= 0 or self.dv <= 0 or not 0 < self.dk <= ops.RECURRENCE_MAX_KEYS:
+            raise AlofaError("unsupported", f"the recurrence kernel takes key sizes up to {ops.RECURRENCE_MAX_KEYS}", f"heads={self.heads} key_dim={self.dk} value_dim={self.dv}")
+
+    def state_need(self):
+        return StateNeed((self.heads, self.dk, self.dv), torch.float32)
+
+    def _leave(self, ctx, o, gate, weight, residual, out):
+        """Head norm, gate and output projection of the read-outs ``o`` (float32 [T, heads * dv])."""
+        y = ctx.scratch("recurrent_gated", (o.shape[0], self.heads * self.dv), self.rt.dtype)
+        ops.headnorm_gate(y, o, gate, weight, self.heads, self.dv, self.eps, self.rt.exact)
+        if out is not None:
+            ops.gemm(out, y, self.w_o, exact=self.rt.exact)
+        else:
+            ops.gemm(residual, y, self.w_o, add_to_out=True, exact=self.rt.exact)
+
+
+class Retention(RecurrentMixer):
+    """params: prefix, hidden, heads, key_dim, value_dim, decay (one per head), position (PartSpec, for heads of
+    key_dim), eps. Tensors: prefix + q, k, v, g, o."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, kd, vd = p["prefix"], p["hidden"], p["heads"] * p["key_dim"], p["heads"] * (p.get("value_dim") or p["key_dim"])
+        return {pre + "q": TensorRule((kd, h), "fan_in"), pre + "k": TensorRule((kd, h), "fan_in"), pre + "v": TensorRule((vd, h), "fan_in"),
+                pre + "g": TensorRule((vd, h), "fan_in"), pre + "o": TensorRule((h, vd), "fan_in")}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p, pre = spec.params, spec.params["prefix"]
+        decay = [float(x) for x in p["decay"]]
+        if len(decay) != self.heads:
+            raise AlofaError("invalid_argument", "retention takes one decay per head", f"heads={self.heads} decays={len(decay)}")
+        if self.dk % 2:
+            raise AlofaError("unsupported", "rotated heads have an even size", f"key_dim={self.dk}")
+        self.decay = torch.tensor(decay, dtype=torch.float32, device=rt.device)
+        self.position = build_part("position", p["position"], weights, rt)
+        order = self.position.channel_order()
+        self.w_in = _stacked(rt, [_heads_in_order(weights[pre + "q"], self.heads, self.dk, order), _heads_in_order(weights[pre + "k"], self.heads, self.dk, order),
+                                  weights[pre + "v"], weights[pre + "g"]])
+        self.w_o = rt.matrix(weights[pre + "o"])
+        self.k_scale = float(self.dk) ** -0.5
+        self.capturable = self.position.table(1) is not None
+
+    def prepare(self, n_positions):
+        self.position.table(n_positions)
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, kd, vd = x.shape[0], self.heads * self.dk, self.heads * self.dv
+        proj = ctx.scratch("recurrent_proj", (T, 2 * kd + 2 * vd), self.rt.dtype)
+        ops.gemm(proj, x, self.w_in, exact=self.rt.exact)
+        table = self.position.table(ctx.n_positions)
+        if table is None:
+            self.position.apply(ctx, proj[:, :kd].unflatten(1, (self.heads, self.dk)), proj[:, kd:2 * kd].unflatten(1, (self.heads, self.dk)))
+        else:      # queries and keys alike: 2 * heads heads to rotate, nothing to write to pages
+            ops.rope_kv_write(proj, table[0], table[1], ctx.positions, 2 * self.heads, 0, self.dk)
+        o = ctx.scratch("recurrent_out", (T, vd), torch.float32)
+        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
+                              self.heads, self.dk, self.dv, ops.DECAY_PER_HEAD, self.decay, k_scale=self.k_scale)
+        self._leave(ctx, o, proj[:, 2 * kd + vd:], None, residual, out)
+
+
+class GatedLinearAttention(RecurrentMixer):
+    """params: prefix, hidden, heads, key_dim, value_dim, tau, rank (of the decay's two-step projection), eps.
+    Tensors: prefix + q, k, v, g, o, a1 [rank, hidden], a2 [heads * key_dim, rank], a2.b, norm [value_dim]."""
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        dv = p.get("value_dim") or p["key_dim"]
+        pre, h, kd, vd, r = p["prefix"], p["hidden"], p["heads"] * p["key_dim"], p["heads"] * dv, p["rank"]
+        return {pre + "q": TensorRule((kd, h), "fan_in"), pre + "k": TensorRule((kd, h), "fan_in"), pre + "v": TensorRule((vd, h), "fan_in"),
+                pre + "g": TensorRule((vd, h), "fan_in"), pre + "o": TensorRule((h, vd), "fan_in"), pre + "norm": TensorRule((dv,), "norm"),
+                pre + "a1": TensorRule((r, h), "fan_in"), pre + "a2": TensorRule((kd, r), "fan_in"), pre + "a2.b": TensorRule((kd,), "decay_bias")}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p, pre = spec.params, spec.params["prefix"]
+        self.tau, self.rank = float(p["tau"]), int(p["rank"])
+        if not self.tau > 0:
+            raise AlofaError("invalid_argument", "tau must be positive", f"tau={self.tau}")
+        self.w_in = _stacked(rt, [weights[pre + n] for n in ("q", "k", "v", "g", "a1")])
+        self.w_a2, self.b_a2 = rt.matrix(weights[pre + "a2"]), rt.vector(weights[pre + "a2.b"])
+        self.w_o = rt.matrix(weights[pre + "o"])
+        self.norm = rt.vector(weights[pre + "norm"].float().repeat(self.heads))      # one weight per value channel, the same for every head
+        self.q_scale = float(self.dk) ** -0.5
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, kd, vd = x.shape[0], self.heads * self.dk, self.heads * self.dv
+        proj = ctx.scratch("recurrent_proj", (T, 2 * kd + 2 * vd + self.rank), self.rt.dtype)
+        ops.gemm(proj, x, self.w_in, exact=self.rt.exact)
+        z = ctx.scratch("recurrent_decay", (T, kd), torch.float32)
+        ops.gemm(z, proj[:, 2 * kd + 2 * vd:], self.w_a2, self.b_a2, exact=self.rt.exact)
+        o = ctx.scratch("recurrent_out", (T, vd), torch.float32)
+        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
+                              self.heads, self.dk, self.dv, ops.DECAY_SIGMOID_ROOT, z, tau=self.tau, q_scale=self.q_scale)
+        self._leave(ctx, o, proj[:, 2 * kd + vd:2 * kd + 2 * vd], self.norm, residual, out)
+
+
+MIXES = ("r", "k", "v", "g", "w")
+
+
+class TokenShift(TimeConv):
+    """out[s] = x + (x' - x) * mu_s for every mix s, x' the row before (zeros before a request's first token); the last
+    row is the part's state per request. params: names (the mu tensors, one per mix), width."""
+    capturable = True
+
+    @classmethod
+    def tensors(cls, spec):
+        return {n: TensorRule((spec.params["width"],), "unit_interval") for n in spec.params["names"]}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.width = int(spec.params["width"])
+        self.mu = rt.vector(torch.stack([weights[n].float() for n in spec.params["names"]]))
+
+    def state_need(self):
+        return StateNeed((1, self.width), self.rt.dtype)
+
+    def forward(self, ctx, where, out, x):
+        state, rows = ctx.state(where), rows_of_requests(ctx)
+        ops.shift_mix(out, x, self.mu, state, rows)
+        ops.keep_last_rows(state, x, rows)
+
+
+class TimeMix(RecurrentMixer):
+    """params: prefix, hidden, heads, key_dim (value heads have the same size), rank (of the decay's two-step
+    projection), eps. Tensors: prefix + mu.r/k/v/g/w, r, k, v, g, o, w1 [rank, hidden], w2 [heads * key_dim, rank], w0,
+    u [heads, key_dim], norm [heads * key_dim]."""
+
+    @classmethod
+    def shift_spec(cls, spec) -> PartSpec:
+        return PartSpec("token_shift", {"names": tuple(spec.params["prefix"] + "mu." + s for s in MIXES), "width": spec.params["hidden"]})
+
+    @classmethod
+    def tensors(cls, spec):
+        p = spec.params
+        pre, h, kd, r = p["prefix"], p["hidden"], p["heads"] * p["key_dim"], p["rank"]
+        out = dict(TokenShift.tensors(cls.shift_spec(spec)))
+        out.update({pre + n: TensorRule((kd, h), "fan_in") for n in ("r", "k", "v", "g")})
+        out.update({pre + "w1": TensorRule((r, h), "fan_in"), pre + "w2": TensorRule((kd, r), "fan_in"), pre + "w0": TensorRule((kd,), "log_rate"),
+                    pre + "u": TensorRule((p["heads"], p["key_dim"]), "bias"), pre + "norm": TensorRule((kd,), "norm"), pre + "o": TensorRule((h, kd), "fan_in")})
+        return out
+
+    def __init__(self, spec, weights, rt):
+        if spec.params.get("value_dim") not in (None, spec.params["key_dim"]):
+            raise AlofaError("invalid_argument", "time mixing has value heads of the key heads' size", f"key_dim={spec.params['key_dim']} value_dim={spec.params['value_dim']}")
+        super().__init__(spec, weights, rt)
+        p, pre = spec.params, spec.params["prefix"]
+        self.rank = int(p["rank"])
+        self.shift = build_part("conv", self.shift_spec(spec), weights, rt)
+        self.w = {n: rt.matrix(weights[pre + n]) for n in ("r", "k", "v", "g", "w1", "w2", "o")}
+        self.w_o = self.w["o"]
+        self.w0, self.norm = rt.vector(weights[pre + "w0"]), rt.vector(weights[pre + "norm"])
+        self.bonus = rt.vector(weights[pre + "u"])
+
+    def stateful_parts(self):
+        return [self, self.shift]
+
+    def forward(self, ctx, where, x, residual, out=None):
+        T, kd = x.shape[0], self.heads * self.dk
+        entry, k = where if isinstance(where, tuple) else (where, 0)
+        exact = self.rt.exact
+        mixes = ctx.scratch("time_mix_inputs", (len(MIXES), T, self.hidden), self.rt.dtype)
+        self.shift.forward(ctx, (entry, k + 1), mixes, x)
+        proj = ctx.scratch("time_mix_proj", (T, 4 * kd), self.rt.dtype)
+        for i, n in enumerate(("r", "k", "v", "g")):
+            ops.gemm(proj[:, i * kd:(i + 1) * kd], mixes[i], self.w[n], exact=exact)
+        low = ctx.scratch("time_mix_low", (T, self.rank), self.rt.dtype)
+        ops.gemm(low, mixes[4], self.w["w1"], exact=exact)
+        ops.activation(low, low, ops.TANH, exact=exact)
+        z = ctx.scratch("recurrent_decay", (T, kd), torch.float32)
+        ops.gemm(z, low, self.w["w2"], self.w0, exact=exact)
+        o = ctx.scratch("recurrent_out", (T, kd), torch.float32)
+        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:3 * kd], ctx.state((entry, k)), rows_of_requests(ctx),
+                              self.heads, self.dk, self.dv, ops.DECAY_EXP_NEG_EXP, z, bonus=self.bonus, before_update=True)
+        self._leave(ctx, o, proj[:, 3 * kd:], self.norm, residual, out)
+
+
+class ParallelMixers(Mixer):
+    """Several mixers side by side that read the same rows; the result is the sum of theirs, each times its scale.
+    params: branches (PartSpecs of mixers that take ``out=``), scales (one per branch), hidden."""
+
+    @classmethod
+    def tensors(cls, spec):
+        from .base import tensors_of
+        out = {}
+        for b in spec.params["branches"]:
+            out.update(tensors_of("mixer", b))
+        return out
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden = int(p["hidden"])
+        self.branches = [build_part("mixer", b, weights, rt) for b in p["branches"]]
+        self.scales = [float(s) for s in p["scales"]]
+        if not self.branches or len(self.scales) != len(self.branches):
+            raise AlofaError("invalid_argument", "one scale per branch, and at least one branch", f"branches={len(self.branches)} scales={len(self.scales)}")
+
+    @property
+    def capturable(self):
+        return all(b.capturable for b in self.branches)
+
+    def stateful_parts(self):
+        return [part for b in self.branches for part in b.stateful_parts()]
+
+    def prepare(self, n_positions):
+        for b in self.branches:
+            b.prepare(n_positions)
+
+    def forward(self, ctx, where, x, residual, out=None):
+        entry, k = where if isinstance(where, tuple) else (where, 0)
+        outs = []
+        for j, b in enumerate(self.branches):
+            buf = ctx.scratch(f"branch_{j}", tuple(residual.shape), torch.float32)
+            b.forward(ctx, (entry, k), x, residual, out=buf)
+            k += len(b.stateful_parts())
+            outs.append(buf)
+        target = residual
+        if out is not None:
+            out.zero_()
+            target = out
+        for j in range(0, len(outs), 2):
+            pair = outs[j:j + 2]
+            ops.add_scaled(target, pair[0], self.scales[j], pair[1] if len(pair) > 1 else None, self.scales[j + 1] if len(pair) > 1 else 0.0, self.rt.exact)
+
+
+register_part("mixer", "retention", Retention)
+register_part("mixer", "gated_linear", GatedLinearAttention)
+register_part("mixer", "time_mix", TimeMix)
+register_part("mixer", "parallel", ParallelMixers)
+register_part("conv", "token_shift", TokenShift)

@@ -2,7 +2,7 @@
 logits; it samples nothing. It drives the engine's own model, step function,
 cache and kernels — the ones generation uses.
 
-    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--blocks N] [--window-blocks N]
+    bin/trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N [--blocks N] [--window-blocks N] [--max-requests N]
 
 Steps come on standard input, one JSON object a line:
 
@@ -47,9 +47,10 @@ class Replayer:
     """The replay loop as an object: one ``step`` per input line."""
 
     def __init__(self, model_dir, dtype: str, max_tokens: int, block_size: int = 16, device: str = "cuda:0",
-                 blocks: Optional[int] = None, window_blocks: Optional[int] = None):
+                 blocks: Optional[int] = None, window_blocks: Optional[int] = None, max_requests: int = 8):
         """``blocks``: pages of every pool (default: what ``max_tokens`` tokens take); ``window_blocks``: pages of
-        the pools of groups of layers that see a window only, when they are to differ."""
+        the pools of groups of layers that see a window only, when they are to differ; ``max_requests``: how many
+        requests can be live at a time (each has a slot for state of fixed size)."""
         from .csrc.build import load
         load()  # compile at the first call if nothing is built; fail loudly if it cannot
         from .cache.manager import CacheManager
@@ -62,7 +63,7 @@ class Replayer:
         if window_blocks is not None:
             n_blocks = {w: n_blocks if w is None else int(window_blocks) for w in CacheManager.windows_of(needs)}
         self.cache = CacheManager(needs, self.model.state_needs(), n_blocks, block_size,
-                                  max_requests=8, device=self.model.rt.device, dtype=self.model.rt.dtype)
+                                  max_requests=int(max_requests), device=self.model.rt.device, dtype=self.model.rt.dtype)
         # the position table is as long as a request can get here, not the checkpoint's
         # max_position_embeddings, which the reference does not read (qwen.mojo:849)
         self.fn = StepFunction(self.model, self.cache, n_positions=max(int(max_tokens), 64))
@@ -131,10 +132,11 @@ def main(argv=None) -> int:
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
     ap.add_argument("--blocks", type=int, default=None, help="pages of the cache pool, instead of what --max-tokens tokens take")
     ap.add_argument("--window-blocks", type=int, default=None, help="pages of the pools of layers that see a window only (default: as the others)")
+    ap.add_argument("--max-requests", type=int, default=4, help="requests that can be live at a time (slots for per-request state)")
     args = ap.parse_args(argv)
     out = Path(args.out)
     out.mkdir(parents=True, exist_ok=True)
-    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size, blocks=args.blocks, window_blocks=args.window_blocks)
+    replayer = Replayer(args.model, args.dtype, args.max_tokens, args.block_size, blocks=args.blocks, window_blocks=args.window_blocks, max_requests=args.max_requests)
     for line in sys.stdin:
         line = line.strip()
         if not line:

@@ -16,7 +16,8 @@ from .safetensors_io import SafeTensorFile
 @dataclass(frozen=True)
 class TensorRule:
     """What a part expects of one tensor. ``init`` names the rule the
-    random-weights mode draws it by: matrix and bias ~ N(0, std), norm ~ 1 + N(0, std).
+    random-weights mode draws it by: matrix and bias ~ N(0, std), norm ~ 1 + N(0, std); the others are listed in
+    ``weights/random_init.py``.
     ``optional`` tensors may be absent (an output matrix tied to the embedding)."""
     shape: tuple
     init: str = "matrix"
