@@ -87,3 +87,16 @@ def tiny_dirs(tmp_path_factory):
         write_random_model(cfg, d, seed=1000 + ord(name))
         out[name] = d
     return out
+
+
+@pytest.fixture(scope="session")
+def tugalix_dirs(tmp_path_factory):
+    """Model folders of the small Tugalix configurations, written by the engine's random-weights mode."""
+    from alofa_amd.weights import write_random_model
+    from tugalix_cases import TUGALIX
+    out = {}
+    for name, cfg in TUGALIX.items():
+        d = tmp_path_factory.mktemp(f"tugalix_{name}")
+        write_random_model(cfg, d, seed=2000 + ord(name))
+        out[name] = d
+    return out
