@@ -26,7 +26,10 @@ tokens per second at the default batch of 8. Beside it:
 chunked prefill; 8 prompts of 16,384 tokens and decoding at batch 32 with a
 context of 4,096) through the same engine and print their own line;
 ``--config 1.5b``, ``3b`` and ``14b`` run the continuous batch at those sizes.
-``--sweep batch`` and ``--sweep context`` take any of the configurations."""
+``--sweep batch`` and ``--sweep context`` take any of the configurations.
+
+``--design tugalix`` measures another design beside Qwen2 at equal sizes: prefill of one prompt and decode steps at
+batch 1, 8 and 64, at a few widths (``--sizes``), a line per point and model."""
 import argparse
 import json
 import statistics
@@ -490,6 +493,59 @@ def sweep(args):
     return 0
 
 
+# ------------------------------------------------------------------- another design beside the closest one
+
+def tugalix_sizes(width, heads, dim, ff, layers, vocab=32000):
+    """A Tugalix model of ``layers`` layers in the order parallel, retention, gated linear attention, retention, every one
+    with a feed-forward, and the Qwen2 model of equal width, heads, layers and feed-forward weights beside it."""
+    kv = max(1, heads // 4)
+    rot = {"dims": dim, "base": 1000000.0}
+    kinds = [("parallel", {"left": {"heads": heads, "kv_heads": kv, "dim": dim, "vdim": dim, "scale": dim ** -0.5, "rot": rot},
+                           "right": {"heads": heads, "dim": dim, "rank": 64}, "left_scale": 1.0, "right_scale": 1.0}),
+             ("retention", {"heads": heads, "dim": dim, "vdim": dim, "rot": rot, "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(heads)]}),
+             ("gla", {"heads": heads, "dim": dim, "vdim": dim, "tau": 16.0, "rank": 16}),
+             ("retention", {"heads": heads, "dim": dim, "vdim": dim, "rot": rot, "decay": [1.0 - 2.0 ** (-5 - i % 8) for i in range(heads)]})]
+    tug = {"architecture": "Tugalix", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "canon": {"taps": 4}, "logit_scale": 1.0,
+           "layers": [{"type": kinds[i % 4][0], "mixer": kinds[i % 4][1], "mlp": {"kind": "dense", "ff": ff}} for i in range(layers)]}
+    qwen = dict(family(layers, width, heads, kv, ff * 2 // 3 // 64 * 64, vocab, False), head_dim=dim)
+    return tug, qwen
+
+
+DESIGN_SIZES = {"1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
+
+
+def designs(args):
+    """Prefill (one prompt of 2,048 tokens in one step) and decode steps (batch 1, 8 and 64 at a context of about 550) of
+    Tugalix beside Qwen2 at equal sizes, random weights: one line per point and model."""
+    sizes = [s for s in (args.sizes.split(",") if args.sizes else DESIGN_SIZES)]
+    for size in sizes:
+        if size not in DESIGN_SIZES:
+            print(f"no such size: {size} (known: {','.join(DESIGN_SIZES)})")
+            return 2
+        for name, cfg in zip(("tugalix", "qwen2"), tugalix_sizes(*DESIGN_SIZES[size])):
+            if args.only and name != args.only:
+                continue
+            cfg = dict(cfg, vocab_size=cfg.get("vocab_size", cfg.get("vocab")))      # (the points draw their tokens by this key)
+            model = device_model({k: v for k, v in cfg.items() if not (name == "tugalix" and k == "vocab_size")}, args.dtype, 20261126)
+            weights = model[1].weight_bytes()
+            if not args.no_prefill:
+                pp = PrefillPoint(model, cfg, args.dtype, T=args.prompt_tokens)
+                pp.run()
+                pre = [pp.run() for _ in range(5)]
+                print(json.dumps({"design": name, "size": size, "point": "prefill", "tokens": args.prompt_tokens, **spread(pre),
+                                  "tok_s": round(args.prompt_tokens / statistics.median(pre), 1)}), flush=True)
+                del pp
+            for batch in (int(b) for b in (args.batches or "1,8,64").split(",")):
+                pt = DecodePoint(model, cfg, args.dtype, batch, PROMPT)
+                pt.run(args.warmup)
+                s = pt.run(args.steps)
+                print(json.dumps({"design": name, "size": size, "point": "decode", "batch": batch, "context": PROMPT, "ms_per_step": round(s * 1e3, 4),
+                                  "tok_s": round(batch / s, 1), "weights_gb_s": round(weights / s / 1e9, 1)}), flush=True)
+                pt.close()
+            del model
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -505,6 +561,11 @@ def main():
     ap.add_argument("--serve", action="store_true", help="the continuous batch of 64 requests (prompts of 128..2,048 tokens, 256 new tokens, chunks of 512) at the sizes of --config")
     ap.add_argument("--batches", default=None, help="with --sweep batch: these batch sizes only (comma-separated), e.g. to profile one point")
     ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
+    ap.add_argument("--design", choices=["tugalix"], default=None, help="prefill and decode of this design beside Qwen2 at equal sizes (--sizes), a line per point")
+    ap.add_argument("--sizes", default=None, help=f"with --design: which of {','.join(DESIGN_SIZES)} (comma-separated; default all)")
+    ap.add_argument("--only", choices=["tugalix", "qwen2"], default=None, help="with --design: this model alone (for profiling)")
+    ap.add_argument("--prompt-tokens", type=int, default=2048, help="with --design: tokens of the prefill point's prompt")
+    ap.add_argument("--no-prefill", action="store_true", help="with --design: decode points only")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this engine has no multi-GPU path (--gpus must be 1)")
@@ -512,6 +573,8 @@ def main():
 
     from alofa_amd.csrc.build import load
     load()
+    if args.design:
+        return designs(args)
     if args.sweep:
         return sweep(args)
     if args.config in ("1.5b", "3b", "7b", "14b") or args.serve:
