@@ -12,6 +12,8 @@
 // State and all arithmetic of the recurrences are float; q, k, v and gates come in the activation type.
 #include "common.h"
 
+#include <type_traits>
+
 namespace alofa {
 
 // ---- short causal convolution ------------------------------------------------------------------------
@@ -67,6 +69,52 @@ __global__ void __launch_bounds__(256) keep_last_rows_kernel(TI* __restrict__ st
     if (i < keep) st[static_cast<int64_t>(i) * width + c] = kept[i];
 }
 
+// Layer norm, convolution and the state's step in one launch, for steps in which every request brings one row (row r is
+// request r): out[r] = n + conv(n) with n = layer norm of x[r] (weight and bias), the rows before it taken from the state,
+// which then moves on by n. A block owns 256 channels of a row (every block of a row takes the row's two sums itself: the
+// row is a few kilobytes), a thread one channel of the request's state: it fetches what the state holds at once, and
+// writes afterwards.
+template <typename TO, typename Acc>
+__global__ void __launch_bounds__(256) norm_conv_step_kernel(TO* __restrict__ out, const float* __restrict__ x, const float* __restrict__ nw,
+                                                             const float* __restrict__ nb, float eps, const float* __restrict__ w,
+                                                             float* __restrict__ state, const int32_t* __restrict__ req_slot, int width, int taps) {
+  __shared__ Acc scratch[4];
+  const int r = blockIdx.y, c = blockIdx.x * 256 + threadIdx.x;
+  const float* src = x + static_cast<int64_t>(r) * width;
+  float* st = state + static_cast<int64_t>(req_slot[r]) * (taps - 1) * width;
+  float kept[kMaxKeep], wc[kMaxKeep + 1];
+#pragma unroll
+  for (int jj = 0; jj < kMaxKeep; ++jj) kept[jj] = (c < width && jj < taps - 1) ? st[static_cast<int64_t>(jj) * width + c] : 0.f;
+#pragma unroll
+  for (int jj = 0; jj <= kMaxKeep; ++jj) wc[jj] = (c < width && jj < taps) ? w[static_cast<int64_t>(c) * taps + jj] : 0.f;
+  Acc s = 0;
+  for (int e = threadIdx.x; e < width; e += 256) s += static_cast<Acc>(src[e]);
+  const Acc mean = block_sum<Acc, 256>(s, scratch) / static_cast<Acc>(width);
+  Acc ss = 0;
+  for (int e = threadIdx.x; e < width; e += 256) {
+    const Acc d = static_cast<Acc>(src[e]) - mean;
+    ss += d * d;
+  }
+  const Acc var = block_sum<Acc, 256>(ss, scratch) / static_cast<Acc>(width);
+  if (c >= width) return;
+  const Acc inv = static_cast<Acc>(1) / sqrt(var + static_cast<Acc>(eps));
+  const float n = static_cast<float>((static_cast<Acc>(src[c]) - mean) * inv * static_cast<Acc>(nw[c]) + static_cast<Acc>(nb[c]));
+  Acc acc = static_cast<Acc>(n);
+  float last = n;      // the filter's own tap on the row itself comes last, as in the kernel for any rows
+#pragma unroll
+  for (int jj = 0; jj < kMaxKeep; ++jj) {
+    if (jj < taps - 1) {
+      acc += static_cast<Acc>(wc[jj]) * static_cast<Acc>(kept[jj]);
+      if (jj > 0) st[static_cast<int64_t>(jj - 1) * width + c] = kept[jj];
+    }
+  }
+#pragma unroll
+  for (int jj = 0; jj <= kMaxKeep; ++jj)
+    if (jj == taps - 1) acc += static_cast<Acc>(wc[jj]) * static_cast<Acc>(last);
+  if (taps > 1) st[static_cast<int64_t>(taps - 2) * width + c] = n;
+  store_f32(out + static_cast<int64_t>(r) * width + c, static_cast<float>(acc));
+}
+
 // ---- mix with the token before --------------------------------------------------------------------------
 // out[s, t, c] = x[t, c] + (x[t-1, c] - x[t, c]) * mu[s, c] for s < n_mixes; the row before a request's first row
 // of this step is state[slot, c] (zeros for a new request). The state is kept by keep_last_rows (keep = 1).
@@ -97,112 +145,202 @@ __global__ void __launch_bounds__(256) shift_mix_kernel(T* __restrict__ out, con
 //   kDecaySigmoidRoot: sigmoid(z)^(1/tau), z = decay_in[t, head * dk + i], formed as exp(log_sigmoid(z) / tau),
 //   kDecayExpNegExp:   exp(-exp(z)).
 //
-// A block owns (request, head, a slice of up to 64 value channels). Lanes are value channels; wave g owns the key channels
-// g * KPT .. g * KPT + KPT - 1 and keeps its share of S in registers (KPT floats per lane). Rows go through LDS in chunks:
-// all threads fetch the chunk's q, k, decays (made once per row and channel, not per lane) and v; then every wave runs the
-// chunk's rows in order against LDS alone, leaving its partial read-outs there; after a barrier they are added over the
-// waves in wave order and written. Within a wave the sum over its key channels runs in ascending order, so a read-out
-// depends on nothing but the rows before it: not on how rows were cut into steps or chunks.
-enum DecayKind : int { kDecayPerHead = 0, kDecaySigmoidRoot = 1, kDecayExpNegExp = 2 };
+// A block owns (request, head, a slice of CW value channels), CW = 16, 32 or 64: the fewer blocks a step has, the narrower
+// the slices, so that a lone prompt still spreads over the chip. A wavefront is 64 / CW groups of CW lanes; lanes of a group
+// are value channels, and group g of wave w owns the KL key channels from (w * groups + g) * KL on and keeps its share of S
+// in registers (KL floats per lane). Rows go through LDS in chunks: all threads fetch the chunk's q, k, decays (made once
+// per row and channel, not per lane) and v; then every wave runs the chunk's rows in order against LDS alone (16-byte
+// reads that a group shares), leaving its groups' partial read-outs there; after a barrier they are added over waves and
+// groups in a fixed order and written. A read-out depends on nothing but the rows before it: not on how rows were cut
+// into steps or chunks.
+enum DecayKind : int { kDecayPerHead = 0, kDecaySigmoidRoot = 1, kDecayExpNegExp = 2, kDecayGiven = 3 };
 
-template <typename T, int KPT>
-__global__ void __launch_bounds__(KPT == 64 ? 512 : 256) linear_recurrence_kernel(
+__device__ __forceinline__ float decay_of(float z, int kind, float inv_tau) {
+  if (kind == kDecaySigmoidRoot) {
+    // log sigmoid(z) = -(max(-z, 0) + log1p(exp(-|z|)))
+    const float ls = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));
+    return expf(ls * inv_tau);
+  }
+  return kind == kDecayExpNegExp ? expf(-expf(z)) : z;
+}
+
+// The decays of many rows, made in place before the recurrence runs (which then takes them as given): a prompt's rows
+// are all there, and making their decays takes the whole chip a few microseconds, where the blocks of the recurrence,
+// few and each bound to its rows' order, would spend more time on them than on the recurrence itself.
+__global__ void __launch_bounds__(256) decay_kernel(float* __restrict__ z, int64_t stride, int64_t rows, int width, int kind, float inv_tau) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * width) return;
+  float* p = z + idx / width * stride + idx % width;
+  *p = decay_of(*p, kind, inv_tau);
+}
+
+template <typename T, int KL, bool kPerHead>
+__global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel(
     float* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
     const T* __restrict__ v, int64_t v_stride, const float* __restrict__ decay_in, int64_t decay_stride, const float* __restrict__ decay_head,
     const float* __restrict__ bonus, float* __restrict__ state, const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off,
-    int heads, int dk, int dv, int decay_kind, float inv_tau, float q_scale, float k_scale, int before_update, int chunk) {
-  extern __shared__ float lds[];
+    int heads, int dk, int dv, int decay_kind, float inv_tau, float q_scale, float k_scale, int before_update, int chunk, int cw_log2) {
+  extern __shared__ float4 lds4[];
+  float* lds = reinterpret_cast<float*>(lds4);
+  const int cw = 1 << cw_log2, groups = kWave >> cw_log2;
   const int n_waves = blockDim.x / kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
-  const int r = blockIdx.z, head = blockIdx.y, j0 = blockIdx.x * kWave;
+  const int col = lane & (cw - 1), group = lane >> cw_log2;
+  const int r = blockIdx.z, head = blockIdx.y, j0 = blockIdx.x * cw;
   const int row0 = row_off ? row_off[r] : r, end = row_off ? row_off[r + 1] : r + 1;
-  const int j = j0 + lane;
+  const int j = j0 + col;
   const bool live = j < dv;
-  const int i0 = wave * KPT;
-  // LDS: q, k, w as [chunk][dk_pad]; v as [chunk][64]; partial read-outs as [chunk][waves][64]
-  const int dk_pad = n_waves * KPT;
+  const int i0 = (wave * groups + group) * KL;
+  // LDS: q, k, w as [chunk][dk_pad]; v as [chunk][cw]; partial read-outs as [chunk][waves * groups][cw]
+  const int dk_pad = n_waves * groups * KL, parts = n_waves * groups;
   float* lq = lds;
   float* lk = lq + chunk * dk_pad;
   float* lw = lk + chunk * dk_pad;
   float* lv = lw + chunk * dk_pad;
-  float* lp = lv + chunk * kWave;
+  float* lp = lv + chunk * cw;
 
   float* S_g = state + ((static_cast<int64_t>(req_slot[r]) * heads + head) * dk) * dv;
-  float S[KPT], u[KPT];
+  float S[KL], u[KL];
 #pragma unroll
-  for (int i = 0; i < KPT; ++i) {
+  for (int i = 0; i < KL; ++i) {
     S[i] = (live && i0 + i < dk) ? S_g[static_cast<int64_t>(i0 + i) * dv + j] : 0.f;
     u[i] = (bonus && i0 + i < dk) ? bonus[head * dk + i0 + i] : 0.f;
   }
-  const float head_decay = decay_kind == kDecayPerHead ? decay_head[head] : 1.f;
+  const float head_decay = kPerHead ? decay_head[head] : 1.f;
 
+  // A chunk's q, k and decay operands are fetched into registers while the chunk before runs (kFetch values of each per
+  // thread), and go to LDS, decays made, once that one's read-outs are written.
+  constexpr int kFetch = 16;      // chunk * dk_pad <= kFetch * threads: the host sees to it
+  T fq[kFetch], fk[kFetch];
+  float fz[kFetch], fv[4];
+  // (value f of a thread is element threadIdx.x + f * threads of the chunk's [rows][dk_pad]: its row and channel follow from
+  // the one before by additions, the only divisions are these)
+  const int threads = blockDim.x;
+  const int first_row = threadIdx.x / dk_pad, first_i = threadIdx.x % dk_pad, step_row = threads / dk_pad, step_i = threads % dk_pad;
+  const int passes = (chunk * dk_pad + threads - 1) / threads, v_passes = ((chunk << cw_log2) + threads - 1) / threads;
+  auto fetch = [&](int c0) {
+    const int n = min(chunk, end - c0);
+    int tt = first_row, i = first_i;
+#pragma unroll
+    for (int f = 0; f < kFetch; ++f) {
+      if (f < passes) {
+        const bool in = tt < n && i < dk;      // (every lane loads: from the chunk's first row and channel where its own is not wanted)
+        const int64_t t = c0 + (in ? tt : 0);
+        const int ch = head * dk + (in ? i : 0);
+        fq[f] = q[t * q_stride + ch];
+        fk[f] = k[t * k_stride + ch];
+        if constexpr (!kPerHead) fz[f] = decay_in[t * decay_stride + ch];
+        i += step_i;
+        tt += step_row;
+        if (i >= dk_pad) i -= dk_pad, ++tt;
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      if (f < v_passes) {
+        const int e = threadIdx.x + f * threads;
+        const int tv = e >> cw_log2, jj = e & (cw - 1);
+        const bool in = tv < n && j0 + jj < dv;
+        fv[f] = load_f32(v + static_cast<int64_t>(c0 + (in ? tv : 0)) * v_stride + head * dv + (in ? j0 + jj : 0));
+        if (!in) fv[f] = 0.f;
+      }
+    }
+  };
+  if (row0 < end) fetch(row0);
   for (int c0 = row0; c0 < end; c0 += chunk) {
     const int n = min(chunk, end - c0);
     __syncthreads();      // the chunk before is written out; LDS is free again
-    for (int e = threadIdx.x; e < n * dk_pad; e += blockDim.x) {
-      const int tt = e / dk_pad, i = e % dk_pad;
-      const int64_t t = c0 + tt;
-      float qv = 0.f, kv = 0.f, wv = 1.f;
-      if (i < dk) {
-        qv = load_f32(q + t * q_stride + head * dk + i) * q_scale;
-        kv = load_f32(k + t * k_stride + head * dk + i) * k_scale;
-        if (decay_kind == kDecayPerHead) {
-          wv = head_decay;
-        } else {
-          const float z = decay_in[t * decay_stride + head * dk + i];
-          if (decay_kind == kDecaySigmoidRoot) {
-            // log sigmoid(z) = -(max(-z, 0) + log1p(exp(-|z|)))
-            const float ls = -(fmaxf(-z, 0.f) + log1pf(expf(-fabsf(z))));
-            wv = expf(ls * inv_tau);
-          } else {
-            wv = expf(-expf(z));
+    {
+      int tt = first_row, i = first_i;
+#pragma unroll
+      for (int f = 0; f < kFetch; ++f) {
+        if (f < passes) {
+          if (tt < n) {
+            const int e = threadIdx.x + f * threads;
+            float qv = 0.f, kv = 0.f, wv = 1.f;
+            if (i < dk) {
+              qv = load_f32(&fq[f]) * q_scale;
+              kv = load_f32(&fk[f]) * k_scale;
+              if constexpr (!kPerHead) wv = decay_of(fz[f], decay_kind, inv_tau);
+            }
+            lq[e] = qv;
+            lk[e] = kv;
+            if constexpr (!kPerHead) lw[e] = wv;
+          }
+          i += step_i;
+          tt += step_row;
+          if (i >= dk_pad) i -= dk_pad, ++tt;
+        }
+      }
+    }
+#pragma unroll
+    for (int f = 0; f < 4; ++f) {
+      const int e = threadIdx.x + f * threads;
+      if (f < v_passes && e < n * cw) lv[e] = fv[f];
+    }
+    __syncthreads();
+    if (c0 + chunk < end) fetch(c0 + chunk);
+    auto run_rows = [&](auto before) {
+      constexpr bool kBefore = decltype(before)::value;
+      // kRows rows at a time: their operands are asked of LDS together, then the rows run in order (a wave is alone on
+      // its SIMD, so what it waits for is not hidden by others)
+      constexpr int kRows = KL <= 8 ? 4 : KL == 16 ? 2 : 1;
+      for (int t0 = 0; t0 < n; t0 += kRows) {
+        float vj[kRows];
+        float4 q4[kRows][KL / 4], k4[kRows][KL / 4], w4[kRows][KL / 4];
+#pragma unroll
+        for (int a = 0; a < kRows; ++a) {
+          const int tt = min(t0 + a, n - 1);
+          vj[a] = lv[tt * cw + col];
+#pragma unroll
+          for (int i = 0; i < KL / 4; ++i) {
+            q4[a][i] = reinterpret_cast<const float4*>(lq + tt * dk_pad + i0)[i];
+            k4[a][i] = reinterpret_cast<const float4*>(lk + tt * dk_pad + i0)[i];
+            if constexpr (!kPerHead) w4[a][i] = reinterpret_cast<const float4*>(lw + tt * dk_pad + i0)[i];
+            else w4[a][i] = make_float4(head_decay, head_decay, head_decay, head_decay);
+          }
+        }
+#pragma unroll
+        for (int a = 0; a < kRows; ++a) {
+          if (t0 + a < n) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < KL; i += 4) {
+              const float qs[4] = {q4[a][i / 4].x, q4[a][i / 4].y, q4[a][i / 4].z, q4[a][i / 4].w};
+              const float ks[4] = {k4[a][i / 4].x, k4[a][i / 4].y, k4[a][i / 4].z, k4[a][i / 4].w};
+              const float ws[4] = {w4[a][i / 4].x, w4[a][i / 4].y, w4[a][i / 4].z, w4[a][i / 4].w};
+#pragma unroll
+              for (int e = 0; e < 4; ++e) {
+                const float kvv = ks[e] * vj[a];
+                if constexpr (kBefore) {
+                  acc[e] += qs[e] * (S[i + e] + u[i + e] * kvv);
+                  S[i + e] = ws[e] * S[i + e] + kvv;
+                } else {
+                  S[i + e] = ws[e] * S[i + e] + kvv;
+                  acc[e] += qs[e] * S[i + e];
+                }
+              }
+            }
+            lp[((t0 + a) * parts + wave * groups + group) * cw + col] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
           }
         }
       }
-      lq[e] = qv;
-      lk[e] = kv;
-      lw[e] = wv;
-    }
-    for (int e = threadIdx.x; e < n * kWave; e += blockDim.x) {
-      const int tt = e / kWave, jj = e % kWave;
-      lv[e] = j0 + jj < dv ? load_f32(v + static_cast<int64_t>(c0 + tt) * v_stride + head * dv + j0 + jj) : 0.f;
-    }
+    };
+    if (before_update) run_rows(std::true_type{});
+    else run_rows(std::false_type{});
     __syncthreads();
-    for (int tt = 0; tt < n; ++tt) {
-      const float vj = lv[tt * kWave + lane];
-      const float* pq = lq + tt * dk_pad + i0;
-      const float* pk = lk + tt * dk_pad + i0;
-      const float* pw = lw + tt * dk_pad + i0;
-      float acc = 0.f;
-      if (before_update) {
-#pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-          const float kvv = pk[i] * vj;
-          acc += pq[i] * (S[i] + u[i] * kvv);
-          S[i] = pw[i] * S[i] + kvv;
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < KPT; ++i) {
-          S[i] = pw[i] * S[i] + pk[i] * vj;
-          acc += pq[i] * S[i];
-        }
-      }
-      lp[(tt * n_waves + wave) * kWave + lane] = acc;
-    }
-    __syncthreads();
-    for (int e = threadIdx.x; e < n * kWave; e += blockDim.x) {
-      const int tt = e / kWave, jj = e % kWave;
+    for (int e = threadIdx.x; e < n * cw; e += blockDim.x) {
+      const int tt = e >> cw_log2, jj = e & (cw - 1);
       if (j0 + jj < dv) {
         float acc = 0.f;
-        for (int g = 0; g < n_waves; ++g) acc += lp[(tt * n_waves + g) * kWave + jj];
+        for (int g = 0; g < parts; ++g) acc += lp[(tt * parts + g) * cw + jj];
         out[(static_cast<int64_t>(c0 + tt) * heads + head) * dv + j0 + jj] = acc;
       }
     }
   }
   if (live) {
 #pragma unroll
-    for (int i = 0; i < KPT; ++i)
+    for (int i = 0; i < KL; ++i)
       if (i0 + i < dk) S_g[static_cast<int64_t>(i0 + i) * dv + j] = S[i];
   }
 }
@@ -229,6 +367,19 @@ extern "C" int alofa_short_conv(void* out, int out_dtype, const void* h, int h_d
   return check_launch("short_conv");
 }
 
+extern "C" int alofa_norm_conv_step(void* out, int out_dtype, const float* x, const float* nw, const float* nb, float eps, const float* w, float* state,
+                                    const int32_t* req_slot, int rows, int width, int taps, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && taps >= 1 && eps > 0.f, "norm_conv_step: bad sizes (rows=%d width=%d taps=%d)", rows, width, taps);
+  ALOFA_REQUIRE(taps - 1 <= kMaxKeep, "norm_conv_step: at most %d taps", kMaxKeep + 1);
+  ALOFA_REQUIRE(!exact || out_dtype == kF32, "norm_conv_step: the exact path writes float32");
+  if (rows == 0) return 0;
+  const dim3 grid((width + 255) / 256, rows);
+  if (exact) norm_conv_step_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), x, nw, nb, eps, w, state, req_slot, width, taps);
+  else if (out_dtype == kF32) norm_conv_step_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), x, nw, nb, eps, w, state, req_slot, width, taps);
+  else norm_conv_step_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), x, nw, nb, eps, w, state, req_slot, width, taps);
+  return check_launch("norm_conv_step");
+}
+
 extern "C" int alofa_keep_last_rows(void* state, const void* h, int dtype, const int32_t* req_slot, const int32_t* row_off, int requests, int width,
                                     int keep, hipStream_t stream) {
   ALOFA_REQUIRE(requests >= 0 && width > 0 && keep >= 0 && keep <= kMaxKeep, "keep_last_rows: bad sizes (requests=%d width=%d keep=%d)", requests, width, keep);
@@ -249,46 +400,72 @@ extern "C" int alofa_shift_mix(void* out, const void* x, int dtype, const float*
   return check_launch("shift_mix");
 }
 
-// Keys per thread and waves for a key size: four waves where that gives a share of 8, 16, 32 or 64 keys, more waves of 64 beyond.
-static inline void recurrence_shape(int dk, int* kpt, int* waves) {
-  const int quarter = (dk + 3) / 4;
-  *kpt = quarter <= 8 ? 8 : quarter <= 16 ? 16 : quarter <= 32 ? 32 : 64;
-  *waves = (dk + *kpt - 1) / *kpt;
+constexpr int kDecayApartFrom = 64;      // steps of more rows make their decays in a launch of their own
+
+// How a launch is shaped: the width of a block's slice of value channels (halved while a step has too few blocks to fill
+// the chip, down to 16), and from it the keys a lane keeps and the waves of a block (four where the key size allows).
+struct RecurrenceShape {
+  int cw_log2, kl, waves;
+};
+static inline RecurrenceShape recurrence_shape(int requests, int heads, int dk, int dv) {
+  int cw_log2 = dv <= 16 ? 4 : dv <= 32 ? 5 : 6;
+  const int64_t want = 2 * static_cast<int64_t>(compute_units());
+  while (cw_log2 > 4 && static_cast<int64_t>(requests) * heads * ((dv + (1 << cw_log2) - 1) >> cw_log2) < want) --cw_log2;
+  const int groups = 64 >> cw_log2;
+  const int share = (dk + 4 * groups - 1) / (4 * groups);
+  const int kl = share <= 4 ? 4 : share <= 8 ? 8 : share <= 16 ? 16 : share <= 32 ? 32 : 64;
+  return {cw_log2, kl, (dk + kl * groups - 1) / (kl * groups)};
 }
 
-extern "C" int alofa_linear_recurrence_lds_bytes(int dk, int chunk) {
-  int kpt, waves;
-  recurrence_shape(dk, &kpt, &waves);
-  return chunk * (3 * waves * kpt + kWave + waves * kWave) * static_cast<int>(sizeof(float));
+static inline int recurrence_lds_bytes(const RecurrenceShape& s, int chunk) {
+  const int groups = 64 >> s.cw_log2;
+  return chunk * (3 * s.waves * groups * s.kl + (1 << s.cw_log2) + s.waves * kWave) * static_cast<int>(sizeof(float));
 }
 
 extern "C" int alofa_linear_recurrence(float* out, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
-                                       int dtype, const float* decay_in, int64_t decay_stride, const float* decay_head, const float* bonus,
-                                       float* state, const int32_t* req_slot, const int32_t* row_off, int requests, int heads, int dk, int dv,
-                                       int decay_kind, float tau, float q_scale, float k_scale, int before_update, int chunk, hipStream_t stream) {
+                                       int dtype, float* decay_in, int64_t decay_stride, const float* decay_head, const float* bonus,
+                                       float* state, const int32_t* req_slot, const int32_t* row_off, int requests, int rows, int heads, int dk, int dv,
+                                       int decay_kind, float tau, float q_scale, float k_scale, int before_update, hipStream_t stream) {
   ALOFA_REQUIRE(requests >= 0 && heads > 0 && dk > 0 && dk <= 512 && dv > 0, "linear_recurrence: bad sizes (requests=%d heads=%d dk=%d dv=%d; dk at most 512)", requests, heads, dk, dv);
-  ALOFA_REQUIRE(decay_kind >= kDecayPerHead && decay_kind <= kDecayExpNegExp, "linear_recurrence: no such kind of decay (%d)", decay_kind);
+  ALOFA_REQUIRE(decay_kind >= kDecayPerHead && decay_kind <= kDecayGiven && rows >= requests, "linear_recurrence: no such kind of decay (%d), or fewer rows than requests", decay_kind);
   ALOFA_REQUIRE(decay_kind == kDecayPerHead ? decay_head != nullptr : decay_in != nullptr, "linear_recurrence: the decay's operand is absent");
   ALOFA_REQUIRE(decay_kind != kDecaySigmoidRoot || tau > 0.f, "linear_recurrence: tau must be positive");
-  ALOFA_REQUIRE(chunk >= 1 && chunk <= 64, "linear_recurrence: rows per chunk lie in 1..64 (%d)", chunk);
   if (requests == 0) return 0;
-  int kpt, waves;
-  recurrence_shape(dk, &kpt, &waves);
-  const int lds = alofa_linear_recurrence_lds_bytes(dk, chunk);
-  ALOFA_REQUIRE(lds <= 64 * 1024, "linear_recurrence: a chunk of %d rows of %d keys does not fit LDS", chunk, dk);
-  const dim3 grid((dv + kWave - 1) / kWave, heads, requests), block(waves * kWave);
-  const float inv_tau = decay_kind == kDecaySigmoidRoot ? 1.f / tau : 0.f;
-#define ALOFA_SCAN(T, KPT) linear_recurrence_kernel<T, KPT><<<grid, block, lds, stream>>>(out, static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, \
-    static_cast<const T*>(v), v_stride, decay_in, decay_stride, decay_head, bonus, state, req_slot, row_off, heads, dk, dv, decay_kind, inv_tau, q_scale, k_scale, before_update, chunk)
-#define ALOFA_SCAN_T(T)                  \
-  switch (kpt) {                         \
-    case 8: ALOFA_SCAN(T, 8); break;     \
-    case 16: ALOFA_SCAN(T, 16); break;   \
-    case 32: ALOFA_SCAN(T, 32); break;   \
-    default: ALOFA_SCAN(T, 64); break;   \
+  if (decay_kind != kDecayPerHead && decay_kind != kDecayGiven && rows > kDecayApartFrom) {
+    const float inv = decay_kind == kDecaySigmoidRoot ? 1.f / tau : 0.f;
+    decay_kernel<<<blocks_of(static_cast<int64_t>(rows) * heads * dk), 256, 0, stream>>>(decay_in, decay_stride, rows, heads * dk, decay_kind, inv);
+    if (check_launch("linear_recurrence (decays)")) return 1;
+    decay_kind = kDecayGiven;
   }
-  if (dtype == kF32) { ALOFA_SCAN_T(float) } else { ALOFA_SCAN_T(bf16_t) }
-#undef ALOFA_SCAN_T
+  const RecurrenceShape shape = recurrence_shape(requests, heads, dk, dv);
+  // rows staged in LDS at a time: sixteen, or as many as 64 KB hold for long keys; one where every request brings a single
+  // row (decoding: little LDS a block, so that many blocks share a compute unit and hide each other's waits)
+  int chunk = rows == requests ? 1 : 16;
+  const int groups = 64 >> shape.cw_log2, threads = shape.waves * kWave;
+  // (... and as a thread's registers fetch ahead: 16 values of q, k and the decay's operand each, 4 of v)
+  while (chunk > 1 && (recurrence_lds_bytes(shape, chunk) > 64 * 1024 || chunk * shape.waves * groups * shape.kl > 16 * threads || (chunk << shape.cw_log2) > 4 * threads)) chunk /= 2;
+  ALOFA_REQUIRE(shape.waves * groups * shape.kl <= 16 * threads, "linear_recurrence: %d keys do not fit a block's registers", dk);
+  const int lds = recurrence_lds_bytes(shape, chunk);
+  ALOFA_REQUIRE(lds <= 64 * 1024 && shape.waves * kWave <= (shape.kl == 64 ? 512 : 256), "linear_recurrence: %d keys do not fit a block", dk);
+  const int cw = 1 << shape.cw_log2;
+  const dim3 grid((dv + cw - 1) / cw, heads, requests), block(shape.waves * kWave);
+  const float inv_tau = decay_kind == kDecaySigmoidRoot ? 1.f / tau : 0.f;
+#define ALOFA_SCAN(T, KL, PH) linear_recurrence_kernel<T, KL, PH><<<grid, block, lds, stream>>>(out, static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, \
+    static_cast<const T*>(v), v_stride, decay_in, decay_stride, decay_head, bonus, state, req_slot, row_off, heads, dk, dv, decay_kind, inv_tau, q_scale, k_scale, before_update, chunk, shape.cw_log2)
+#define ALOFA_SCAN_K(T, PH)                  \
+  switch (shape.kl) {                        \
+    case 4: ALOFA_SCAN(T, 4, PH); break;     \
+    case 8: ALOFA_SCAN(T, 8, PH); break;     \
+    case 16: ALOFA_SCAN(T, 16, PH); break;   \
+    case 32: ALOFA_SCAN(T, 32, PH); break;   \
+    default: ALOFA_SCAN(T, 64, PH); break;   \
+  }
+  if (dtype == kF32) {
+    if (decay_kind == kDecayPerHead) { ALOFA_SCAN_K(float, true) } else { ALOFA_SCAN_K(float, false) }
+  } else {
+    if (decay_kind == kDecayPerHead) { ALOFA_SCAN_K(bf16_t, true) } else { ALOFA_SCAN_K(bf16_t, false) }
+  }
+#undef ALOFA_SCAN_K
 #undef ALOFA_SCAN
   return check_launch("linear_recurrence");
 }

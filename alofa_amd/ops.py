@@ -1021,6 +1021,26 @@ def short_conv(out: torch.Tensor, h: torch.Tensor, w: torch.Tensor, state: torch
           _ptr(rows.req_of_row), _I(T), _I(width), _I(taps), _I(int(exact)), _stream())
 
 
+def norm_conv_step(out: torch.Tensor, x: torch.Tensor, norm_w: torch.Tensor, norm_b: torch.Tensor, eps: float, w: torch.Tensor,
+                   state: torch.Tensor, rows: RowsOfRequests, exact: bool = False) -> None:
+    """``layernorm``, ``short_conv`` and ``keep_last_rows`` in one launch for a step in which every request brings one row:
+    out[r] = n + conv(n), n the layer norm of x[r]; the state (float32 [slots, taps - 1, width]) moves on by n."""
+    _gpu("out", out, None, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 2), _gpu("state", state, torch.float32, 3)
+    _gpu("norm_w", norm_w, torch.float32, 1), _gpu("norm_b", norm_b, torch.float32, 1)
+    for n, t in (("out", out), ("x", x), ("w", w), ("state", state), ("norm_w", norm_w), ("norm_b", norm_b)):
+        _contig(n, t)
+    T, width = x.shape
+    taps = w.shape[1]
+    if (tuple(out.shape) != (T, width) or w.shape[0] != width or tuple(state.shape[1:]) != (taps - 1, width) or norm_w.shape[0] != width or norm_b.shape[0] != width
+            or rows.offsets is not None or rows.rows != T or not 1 <= taps <= CONV_MAX_TAPS):
+        raise AlofaError("shape_mismatch", "norm and convolution operands do not fit (one row per request)", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)} state={tuple(state.shape)}")
+    rows.fits("state", state)
+    if exact and out.dtype is not torch.float32:
+        raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
+    _call("alofa_norm_conv_step", _ptr(out), _I(dtype_code(out)), _ptr(x), _ptr(norm_w), _ptr(norm_b), _F(eps), _ptr(w), _ptr(state), _ptr(rows.slots),
+          _I(T), _I(width), _I(taps), _I(int(exact)), _stream())
+
+
 def keep_last_rows(state: torch.Tensor, h: torch.Tensor, rows: RowsOfRequests) -> None:
     """state[slot] [keep, width] = the last ``keep`` rows its request has seen once this step's rows ``h`` are in (older
     ones from the state itself where the step brought fewer)."""
@@ -1045,20 +1065,8 @@ def shift_mix(out: torch.Tensor, x: torch.Tensor, mu: torch.Tensor, state: torch
           _I(T), _I(width), _I(mu.shape[0]), _stream())
 
 
-DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP = 0, 1, 2
+DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP, DECAY_GIVEN = 0, 1, 2, 3
 RECURRENCE_MAX_KEYS = 512
-
-
-def recurrence_chunk(dk: int) -> int:
-    """Rows that the recurrence kernel stages in LDS at a time: sixteen, or as many as 64 KB hold for long keys."""
-    chunk = 16
-    while chunk > 1 and _recurrence_lds(dk, chunk) > 64 * 1024:
-        chunk //= 2
-    return chunk
-
-
-def _recurrence_lds(dk: int, chunk: int) -> int:
-    return int(load().alofa_linear_recurrence_lds_bytes(_I(dk), _I(chunk)))
 
 
 def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests,
@@ -1069,7 +1077,8 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
     [slots, heads, dk, dv] is read and left in ``state``. q, k [T, heads * dk] and v [T, heads * dv] are rows in one
     dtype (row strides allowed); ``out`` float32 [T, heads * dv]. The decay w_t: ``DECAY_PER_HEAD`` with ``decay``
     float32 [heads]; ``DECAY_SIGMOID_ROOT`` sigmoid(z)^(1/tau) or ``DECAY_EXP_NEG_EXP`` exp(-exp(z)) with ``decay`` = z
-    float32 [T, heads * dk] rows."""
+    float32 [T, heads * dk] rows, which a step of many rows overwrites with the decays made of them; ``DECAY_GIVEN``:
+    ``decay`` holds the w_t themselves."""
     _gpu("out", out, torch.float32, 2), _contig("out", out), _gpu("q", q, None, 2), _gpu("k", k, q.dtype, 2), _gpu("v", v, q.dtype, 2)
     _gpu("state", state, torch.float32, 4), _contig("state", state)
     T = q.shape[0]
@@ -1082,7 +1091,7 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
     _gpu("decay", decay, torch.float32, 1 if per_head else 2)
     if per_head:
         _contig("decay", decay)
-    if (tuple(decay.shape) != (heads,)) if per_head else (tuple(decay.shape) != (T, heads * dk)) or decay_kind not in (DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP):
+    if (tuple(decay.shape) != (heads,)) if per_head else (tuple(decay.shape) != (T, heads * dk)) or decay_kind not in (DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP, DECAY_GIVEN):
         raise AlofaError("shape_mismatch", "the decay does not fit its kind", f"decay={tuple(decay.shape)} kind={decay_kind} heads={heads} dk={dk}")
     if bonus is not None:
         _gpu("bonus", bonus, torch.float32, 2), _contig("bonus", bonus)
@@ -1090,5 +1099,5 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
             raise AlofaError("shape_mismatch", "the bonus is [heads, dk] and goes with the read-out before the update", f"bonus={tuple(bonus.shape)}")
     _call("alofa_linear_recurrence", _ptr(out), _ptr(q), _L(_rows("q", q)), _ptr(k), _L(_rows("k", k)), _ptr(v), _L(_rows("v", v)), _I(dtype_code(q)),
           _ptr(None if per_head else decay), _L(0 if per_head else _rows("decay", decay)), _ptr(decay if per_head else None), _ptr(bonus), _ptr(state),
-          _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(heads), _I(dk), _I(dv), _I(decay_kind), _F(tau), _F(q_scale), _F(k_scale),
-          _I(int(before_update)), _I(recurrence_chunk(dk)), _stream())
+          _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(T), _I(heads), _I(dk), _I(dv), _I(decay_kind), _F(tau), _F(q_scale), _F(k_scale),
+          _I(int(before_update)), _stream())

@@ -182,6 +182,11 @@ class TimeConv(Part):
     def prepare(self, n_positions: int) -> None:
         pass
 
+    def fuses_norm(self, ctx, norm) -> bool:
+        """Whether, in this step, the filter would rather apply ``norm`` to the stream itself, in the same launch. A filter
+        that says yes is called as ``forward(ctx, where, out, stream, norm=norm)``."""
+        return False
+
     def forward(self, ctx, where, out: torch.Tensor, x: torch.Tensor) -> None:
         raise NotImplementedError
 
@@ -255,6 +260,10 @@ class Norm(Part):
     def as_rmsnorm(self):
         """(weight float32 [width], eps) when the norm is x / sqrt(mean(x^2) + eps) * weight, which
         some kernels can apply on their way; None for any other norm."""
+        return None
+
+    def as_layernorm(self):
+        """(weight, bias, eps), float32 vectors, when the norm is (x - mean) / sqrt(var + eps) * weight + bias; None otherwise."""
         return None
 
     def forward(self, out: torch.Tensor, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:

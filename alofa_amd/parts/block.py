@@ -132,6 +132,9 @@ class FilteredPreNormBlock(Block):
         if conv is None:
             self.norms[sub].forward(rows, hidden)
             return rows
+        if conv.fuses_norm(ctx, self.norms[sub]):
+            conv.forward(ctx, (entry, self._stateful.index(conv)), rows, hidden, norm=self.norms[sub])
+            return rows
         wide = ctx.scratch("normed_f32", tuple(hidden.shape), torch.float32)
         self.norms[sub].forward(wide, hidden)
         conv.forward(ctx, (entry, self._stateful.index(conv)), rows, wide)

@@ -32,8 +32,16 @@ class ShortCausalConv(TimeConv):
     def state_need(self):
         return StateNeed((self.taps - 1, self.width), torch.float32) if self.taps > 1 else None
 
-    def forward(self, ctx, where, out, x):
-        """out = x + conv(x) for float32 rows x; the state moves on by this step's rows."""
+    def fuses_norm(self, ctx, norm):
+        # single rows (decoding): norm, filter and the state's step are one launch
+        return ctx.max_q_len == 1 and self.taps > 1 and norm.as_layernorm() is not None
+
+    def forward(self, ctx, where, out, x, norm=None):
+        """out = x + conv(x) for float32 rows x (with ``norm``: for the norm of the rows x); the state moves on by this step's rows."""
+        if norm is not None:
+            weight, bias, eps = norm.as_layernorm()
+            ops.norm_conv_step(out, x, weight, bias, eps, self.weight, ctx.state(where), rows_of_requests(ctx), self.rt.exact)
+            return
         if self.taps == 1:      # a filter of one tap sees the row itself only
             state = ctx.scratch("conv_no_state", (ctx.fn.cache.max_requests, 0, self.width), torch.float32)
             ops.short_conv(out, x, self.weight, state, rows_of_requests(ctx), self.rt.exact)

@@ -49,6 +49,9 @@ class LayerNorm(Norm):
         self.weight = rt.vector(weights[spec.params["name"]])
         self.bias = rt.vector(weights[spec.params["bias"]])
 
+    def as_layernorm(self):
+        return self.weight, self.bias, self.eps
+
     def forward(self, out, x, rows=None):
         ops.layernorm(out, x, self.weight, self.bias, self.eps, self.rt.exact, rows)
 

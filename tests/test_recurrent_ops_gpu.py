@@ -115,7 +115,7 @@ def test_linear_recurrence(heads, dk, dv, kind, dtype):
     """Two requests side by side in unequal portions (single rows among them) against the plain recurrence of each."""
     from alofa_amd import ops
     rng = np.random.default_rng(dk + dv)
-    n_slots, T = 4, {3: 41, 0: 29}
+    n_slots, T = 4, {3: 141, 0: 29}      # (steps of more than 64 rows make their decays in a launch of their own)
     data = {}
     for s, n in T.items():
         q, k, v = rng.normal(0, 1, (n, heads * dk)), rng.normal(0, 1, (n, heads * dk)), rng.normal(0, 1, (n, heads * dv))
@@ -139,7 +139,7 @@ def test_linear_recurrence(heads, dk, dv, kind, dtype):
                                   for i in range(heads)], axis=1)
     state = torch.zeros(n_slots, heads, dk, dv, device=DEV)
     state[1] = 3.0
-    parts = {3: cuts(41, (1, 17, 1, 2, 20, 5)), 0: cuts(29, (6, 1, 1, 16, 2, 9))}
+    parts = {3: cuts(141, (1, 17, 1, 2, 100, 5, 15)), 0: cuts(29, (6, 1, 1, 16, 2, 9))}
     got = {3: [], 0: []}
     code = {"per_head": ops.DECAY_PER_HEAD, "sigmoid_root": ops.DECAY_SIGMOID_ROOT, "exp_neg_exp": ops.DECAY_EXP_NEG_EXP}[kind]
     for step in range(max(len(p) for p in parts.values())):
@@ -231,3 +231,23 @@ def test_part_of_a_head_rotated():
     ops.rope_kv_write(both, cos, sin, torch.arange(T, dtype=torch.int32, device=DEV), 2 * heads, 0, d)
     got = both.cpu().numpy().astype(np.float64).reshape(T, 2, heads, d)
     assert np.abs(np.einsum("thd,shd->hts", got[:, 0], got[:, 1]) - want).max() <= 1e-4
+
+
+@pytest.mark.parametrize("taps", [2, 4])
+@pytest.mark.parametrize("exact", [True, False])
+def test_norm_filter_and_state_in_one_launch(taps, exact):
+    """Single rows of three requests: the fused kernel against norm, filter and state update one after the other."""
+    from alofa_amd import ops
+    rng = np.random.default_rng(taps)
+    width, n_slots = 200, 5
+    w, nw, nb = dev(rng.normal(0, 0.5, (width, taps))), dev(rng.normal(1, 0.2, width)), dev(rng.normal(0, 0.3, width))
+    fused, apart = torch.zeros(n_slots, taps - 1, width, device=DEV), torch.zeros(n_slots, taps - 1, width, device=DEV)
+    rows = rows_of([(4, 1), (0, 1), (2, 1)], n_slots)
+    for _ in range(6):
+        x = dev(rng.normal(1.0, 2.0, (3, width)))
+        normed, want, got = torch.empty(3, width, device=DEV), torch.empty(3, width, device=DEV), torch.empty(3, width, device=DEV)
+        ops.layernorm(normed, x, nw, nb, 1e-5, exact)
+        ops.short_conv(want, normed, w, apart, rows, exact)
+        ops.keep_last_rows(apart, normed, rows)
+        ops.norm_conv_step(got, x, nw, nb, 1e-5, w, fused, rows, exact)
+        assert torch.equal(got, want) and torch.equal(fused, apart)

@@ -143,7 +143,6 @@ def test_a_far_key_that_decides(tugalix_dirs, tmp_path, dtype):
     def sharpen(w):
         w["l1.mix.left.q"] *= 6.0
         w["l1.mix.left.k"] *= 6.0
-        w["l1.mix.left.v"] *= 3.0
     d = _rewrite(tugalix_dirs[name], tmp_path / "sharp", sharpen)
     ids = ids_of(name, seed=21, n=330)
     cfg, w = plain_model(str(d))
