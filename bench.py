@@ -535,7 +535,7 @@ def designs(args):
                 print(json.dumps({"design": name, "size": size, "point": "prefill", "tokens": args.prompt_tokens, **spread(pre),
                                   "tok_s": round(args.prompt_tokens / statistics.median(pre), 1)}), flush=True)
                 del pp
-            for batch in (int(b) for b in (args.batches or "1,8,64").split(",")):
+            for batch in (int(b) for b in (args.batches or "1,8,64").split(",") if int(b) > 0):      # (--batches 0: the prefill point alone)
                 pt = DecodePoint(model, cfg, args.dtype, batch, PROMPT)
                 pt.run(args.warmup)
                 s = pt.run(args.steps)
