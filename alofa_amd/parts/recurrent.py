@@ -21,7 +21,8 @@ from .. import ops
 from ..config.base import PartSpec
 from ..errors import AlofaError
 from ..weights.loader import TensorRule
-from .base import Mixer, StateNeed, TimeConv, build_part, register_part
+from .attention import _padded_heads
+from .base import Mixer, StateNeed, TimeConv, build_part, part_class, register_part
 from .rows import rows_of_requests
 
 
@@ -29,13 +30,6 @@ def _stacked(rt, mats: list) -> torch.Tensor:
     if len({m.dtype for m in mats}) > 1:
         mats = [m.float() for m in mats]
     return rt.matrix(torch.cat(mats, dim=0))
-
-
-def _heads_in_order(t: torch.Tensor, heads: int, size: int, order) -> torch.Tensor:
-    if order is None:
-        return t
-    rest = tuple(t.shape[1:])
-    return t.reshape(heads, size, *rest)[:, torch.tensor(order, dtype=torch.long)].reshape(heads * size, *rest).contiguous()
 
 
 class RecurrentMixer(Mixer):
@@ -81,15 +75,18 @@ class Retention(RecurrentMixer):
         decay = [float(x) for x in p["decay"]]
         if len(decay) != self.heads:
             raise AlofaError("invalid_argument", "retention takes one decay per head", f"heads={self.heads} decays={len(decay)}")
-        if self.dk % 2:
-            raise AlofaError("unsupported", "rotated heads have an even size", f"key_dim={self.dk}")
         self.decay = torch.tensor(decay, dtype=torch.float32, device=rt.device)
-        self.position = build_part("position", p["position"], weights, rt)
+        self.k_scale = float(self.dk) ** -0.5
+        # the rotation pairs channels, so a head of odd size gets one more key channel whose q and k are zero (it adds nothing to any product)
+        position, true_dk = p["position"], self.dk
+        if self.dk % 2:
+            self.dk += 1
+            position = part_class("position", position.kind).for_head(position, self.dk)
+        self.position = build_part("position", position, weights, rt)
         order = self.position.channel_order()
-        self.w_in = _stacked(rt, [_heads_in_order(weights[pre + "q"], self.heads, self.dk, order), _heads_in_order(weights[pre + "k"], self.heads, self.dk, order),
+        self.w_in = _stacked(rt, [_padded_heads(weights[pre + "q"], self.heads, true_dk, self.dk, order), _padded_heads(weights[pre + "k"], self.heads, true_dk, self.dk, order),
                                   weights[pre + "v"], weights[pre + "g"]])
         self.w_o = rt.matrix(weights[pre + "o"])
-        self.k_scale = float(self.dk) ** -0.5
         self.capturable = self.position.table(1) is not None
 
     def prepare(self, n_positions):

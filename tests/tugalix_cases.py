@@ -42,6 +42,13 @@ TUGALIX = {
         ("retention", _retention(2, 64, 128, 64, 10000.0, [0.96, 0.995]), None),
         ("parallel", _parallel(2, 2, 128, 128, 128, 1000000.0, 0.09, 4, 64, 16, 0.5, 0.5), None),
         ("gla", {"heads": 2, "dim": 128, "vdim": 128, "tau": 16.0, "rank": 16}, 256)]),
+    # nothing a multiple of eight: width 100, odd head sizes (15 with 6 channels rotated, 9, 7), ranks 7 and 1, five taps, two kv heads of five
+    "E": _config(301, 100, 1e-4, 5, 0.75, [
+        ("retention", _retention(5, 15, 9, 6, 20000.0, [0.7, 0.9, 0.95, 0.99, 1.0]), 150),
+        ("parallel", _parallel(10, 2, 20, 12, 10, 300.0, 0.4, 5, 7, 1, 0.3, 2.0), None),
+        ("parallel", _parallel(1, 1, 30, 50, 30, 10000.0, 0.2, 1, 33, 7, 1.0, 1.0), 66),
+        ("gla", {"heads": 3, "dim": 9, "vdim": 15, "tau": 2.5, "rank": 7}, None),
+        ("gla", {"heads": 1, "dim": 21, "vdim": 100, "tau": 30.0, "rank": 2}, 30)]),
 }
 
 
