@@ -46,16 +46,29 @@ __global__ void __launch_bounds__(256) layernorm_kernel(TO* __restrict__ out, co
 template <typename T, typename Acc>
 __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out, int64_t out_stride, const float* __restrict__ o,
                                                             const T* __restrict__ g, int64_t g_stride, const float* __restrict__ w,
-                                                            int tokens, int heads, int dv, float eps, float out_scale) {
+                                                            int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride) {
   const int64_t unit = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (unit >= static_cast<int64_t>(tokens) * heads) return;
   const int lane = threadIdx.x % kWave;
   const int t = static_cast<int>(unit / heads), h = static_cast<int>(unit % heads);
   const float* src = o + (static_cast<int64_t>(t) * heads + h) * dv;
+  // (o may come in parts, left by blocks that each held a share of the key channels: they are added here, in their order)
+  constexpr int kOwn = 4;      // values a lane keeps between the sum of squares and the scaling (heads up to 256 wide; wider ones are added again)
+  float own[kOwn];
   Acc ss = 0;
-  for (int j = lane; j < dv; j += kWave) {
-    const Acc v = static_cast<Acc>(src[j]);
-    ss += v * v;
+#pragma unroll
+  for (int c = 0; c < kOwn; ++c) {
+    const int j = lane + c * kWave;
+    float v = 0.f;
+    if (j < dv)
+      for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    own[c] = v;
+    ss += static_cast<Acc>(v) * static_cast<Acc>(v);
+  }
+  for (int j = lane + kOwn * kWave; j < dv; j += kWave) {
+    float v = 0.f;
+    for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    ss += static_cast<Acc>(v) * static_cast<Acc>(v);
   }
   ss = wave_sum(ss);
   const Acc inv = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(dv) + static_cast<Acc>(eps));
@@ -64,7 +77,15 @@ __global__ void __launch_bounds__(256) headnorm_gate_kernel(T* __restrict__ out,
   for (int j = lane; j < dv; j += kWave) {
     const Acc z = static_cast<Acc>(load_f32(gate + j));
     const Acc silu = z / (static_cast<Acc>(1) + exp(-z));
-    Acc y = static_cast<Acc>(src[j]) * inv;
+    float v = 0.f;
+    if (j < kOwn * kWave) {
+#pragma unroll
+      for (int c = 0; c < kOwn; ++c)
+        if (j == lane + c * kWave) v = own[c];
+    } else {
+      for (int p = 0; p < parts; ++p) v += src[p * part_stride + j];
+    }
+    Acc y = static_cast<Acc>(v) * inv;
     if (w) y *= static_cast<Acc>(w[h * dv + j]);
     store_f32(dst + j, static_cast<float>(y * silu * static_cast<Acc>(out_scale)));
   }
@@ -141,14 +162,14 @@ extern "C" int alofa_layernorm(void* out, int out_dtype, const float* x, const f
 }
 
 extern "C" int alofa_headnorm_gate(void* out, int64_t out_stride, const float* o, const void* g, int64_t g_stride, int dtype, const float* w,
-                                   int tokens, int heads, int dv, float eps, float out_scale, int exact, hipStream_t stream) {
-  ALOFA_REQUIRE(tokens >= 0 && heads > 0 && dv > 0 && eps > 0.f, "headnorm_gate: bad sizes (tokens=%d heads=%d dv=%d)", tokens, heads, dv);
+                                   int tokens, int heads, int dv, float eps, float out_scale, int parts, int64_t part_stride, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens >= 0 && heads > 0 && dv > 0 && eps > 0.f && parts >= 1, "headnorm_gate: bad sizes (tokens=%d heads=%d dv=%d)", tokens, heads, dv);
   ALOFA_REQUIRE(!exact || dtype == kF32, "headnorm_gate: the exact path is float32");
   if (tokens == 0) return 0;
   const unsigned grid = static_cast<unsigned>((static_cast<int64_t>(tokens) * heads + 3) / 4);
-  if (exact) headnorm_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale);
-  else if (dtype == kF32) headnorm_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale);
-  else headnorm_gate_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, o, static_cast<const bf16_t*>(g), g_stride, w, tokens, heads, dv, eps, out_scale);
+  if (exact) headnorm_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
+  else if (dtype == kF32) headnorm_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, o, static_cast<const float*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
+  else headnorm_gate_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, o, static_cast<const bf16_t*>(g), g_stride, w, tokens, heads, dv, eps, out_scale, parts, part_stride);
   return check_launch("headnorm_gate");
 }
 

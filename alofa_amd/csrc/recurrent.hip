@@ -174,29 +174,56 @@ __global__ void __launch_bounds__(256) decay_kernel(float* __restrict__ z, int64
   *p = decay_of(*p, kind, inv_tau);
 }
 
-template <typename T, int KL, bool kPerHead>
-__global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel(
+// v of lane kLane of the caller's row of 16 lanes, for every lane of the row (a data-parallel-primitive move, which the
+// compiler folds into the multiply that uses it).
+template <int kLane>
+__device__ __forceinline__ float row_lane(float v) {
+  return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), 0x150 + kLane, 0xf, 0xf, true));      // row_newbcast:kLane
+}
+
+template <int kFrom, int kTo, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  if constexpr (kFrom < kTo) {
+    f(std::integral_constant<int, kFrom>{});
+    static_for<kFrom + 1, kTo>(f);
+  }
+}
+
+// What a group needs of one row, q then k then (unless the decay is the head's) w of its KL key channels, lies in LDS as one
+// run of floats; a lane reads the floats r, r + 16, ... (r its place in its row of 16 lanes) and the lanes of the row hand
+// them to one another. Runs begin an odd multiple of 16 floats apart, so that the rows of a wave read different banks.
+template <int KL, bool kPerHead>
+struct RunOfOperands {
+  static constexpr int kFloats = (kPerHead ? 2 : 3) * KL;
+  static constexpr int kLoads = (kFloats + 15) / 16;
+  static constexpr int kStride = 16 * (kLoads | 1);
+};
+
+template <typename T, int KL, bool kPerHead, bool kDirect>
+__global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recurrence_kernel(
     float* __restrict__ out, const T* __restrict__ q, int64_t q_stride, const T* __restrict__ k, int64_t k_stride,
     const T* __restrict__ v, int64_t v_stride, const float* __restrict__ decay_in, int64_t decay_stride, const float* __restrict__ decay_head,
     const float* __restrict__ bonus, float* __restrict__ state, const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off,
-    int heads, int dk, int dv, int decay_kind, float inv_tau, float q_scale, float k_scale, int before_update, int chunk, int cw_log2) {
+    int heads, int dk, int dv, int decay_kind, float inv_tau, float q_scale, float k_scale, int before_update, int chunk, int cw_log2,
+    int key_blocks, int64_t part_stride) {
   extern __shared__ float4 lds4[];
   float* lds = reinterpret_cast<float*>(lds4);
   const int cw = 1 << cw_log2, groups = kWave >> cw_log2;
   const int n_waves = blockDim.x / kWave;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), lane = threadIdx.x % kWave;
   const int col = lane & (cw - 1), group = lane >> cw_log2;
-  const int r = blockIdx.z, head = blockIdx.y, j0 = blockIdx.x * cw;
+  // (with key_blocks > 1 the key channels of a head are dealt out over so many blocks, each with its share of the state's rows;
+  // block kb leaves its part of every read-out in out + kb * part_stride, and whoever reads them adds the parts)
+  const int r = blockIdx.z, head = blockIdx.y / key_blocks, kb = blockIdx.y % key_blocks, j0 = blockIdx.x * cw;
   const int row0 = row_off ? row_off[r] : r, end = row_off ? row_off[r + 1] : r + 1;
   const int j = j0 + col;
   const bool live = j < dv;
-  const int i0 = (wave * groups + group) * KL;
-  // LDS: q, k, w as [chunk][dk_pad]; v as [chunk][cw]; partial read-outs as [chunk][waves * groups][cw]
-  const int dk_pad = n_waves * groups * KL, parts = n_waves * groups;
-  float* lq = lds;
-  float* lk = lq + chunk * dk_pad;
-  float* lw = lk + chunk * dk_pad;
-  float* lv = lw + chunk * dk_pad;
+  // LDS: the groups' runs of operands as [chunk][waves * groups][kStride]; v as [chunk][cw]; partial read-outs as [chunk][waves * groups][cw]
+  using Run = RunOfOperands<KL, kPerHead>;
+  const int dk_pad = n_waves * groups * KL, parts = n_waves * groups, part = wave * groups + group;      // (dk_pad: the key channels of this block)
+  const int key0 = kb * dk_pad, i0 = key0 + part * KL;      // the block's first key channel, and this lane's
+  float* lx = lds;
+  float* lv = lx + chunk * parts * Run::kStride;
   float* lp = lv + chunk * cw;
 
   float* S_g = state + ((static_cast<int64_t>(req_slot[r]) * heads + head) * dk) * dv;
@@ -224,9 +251,9 @@ __global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel
 #pragma unroll
     for (int f = 0; f < kFetch; ++f) {
       if (f < passes) {
-        const bool in = tt < n && i < dk;      // (every lane loads: from the chunk's first row and channel where its own is not wanted)
+        const bool in = tt < n && key0 + i < dk;      // (every lane loads: from the chunk's first row and channel where its own is not wanted)
         const int64_t t = c0 + (in ? tt : 0);
-        const int ch = head * dk + (in ? i : 0);
+        const int ch = head * dk + (in ? key0 + i : 0);
         fq[f] = q[t * q_stride + ch];
         fk[f] = k[t * k_stride + ch];
         if constexpr (!kPerHead) fz[f] = decay_in[t * decay_stride + ch];
@@ -256,16 +283,16 @@ __global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel
       for (int f = 0; f < kFetch; ++f) {
         if (f < passes) {
           if (tt < n) {
-            const int e = threadIdx.x + f * threads;
             float qv = 0.f, kv = 0.f, wv = 1.f;
-            if (i < dk) {
+            if (key0 + i < dk) {
               qv = load_f32(&fq[f]) * q_scale;
               kv = load_f32(&fk[f]) * k_scale;
               if constexpr (!kPerHead) wv = decay_of(fz[f], decay_kind, inv_tau);
             }
-            lq[e] = qv;
-            lk[e] = kv;
-            if constexpr (!kPerHead) lw[e] = wv;
+            float* run = lx + (tt * parts + i / KL) * Run::kStride + i % KL;
+            run[0] = qv;
+            run[KL] = kv;
+            if constexpr (!kPerHead) run[2 * KL] = wv;
           }
           i += step_i;
           tt += step_row;
@@ -284,44 +311,50 @@ __global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel
       constexpr bool kBefore = decltype(before)::value;
       // kRows rows at a time: their operands are asked of LDS together, then the rows run in order (a wave is alone on
       // its SIMD, so what it waits for is not hidden by others)
-      constexpr int kRows = KL <= 8 ? 4 : KL == 16 ? 2 : 1;
+      constexpr int kRows = kDirect ? (KL <= 8 ? 4 : KL == 16 ? 2 : 1) : (KL <= 16 ? 4 : KL == 32 ? 2 : 1);
       for (int t0 = 0; t0 < n; t0 += kRows) {
-        float vj[kRows];
-        float4 q4[kRows][KL / 4], k4[kRows][KL / 4], w4[kRows][KL / 4];
+        float vj[kRows], x[kRows][kDirect ? Run::kFloats : Run::kLoads];
 #pragma unroll
         for (int a = 0; a < kRows; ++a) {
           const int tt = min(t0 + a, n - 1);
           vj[a] = lv[tt * cw + col];
+          if constexpr (kDirect) {      // the wave is one group: every lane reads the whole run (reads of one address, 16 bytes at a time)
+            const float4* run = reinterpret_cast<const float4*>(lx + (tt * parts + part) * Run::kStride);
 #pragma unroll
-          for (int i = 0; i < KL / 4; ++i) {
-            q4[a][i] = reinterpret_cast<const float4*>(lq + tt * dk_pad + i0)[i];
-            k4[a][i] = reinterpret_cast<const float4*>(lk + tt * dk_pad + i0)[i];
-            if constexpr (!kPerHead) w4[a][i] = reinterpret_cast<const float4*>(lw + tt * dk_pad + i0)[i];
-            else w4[a][i] = make_float4(head_decay, head_decay, head_decay, head_decay);
+            for (int m = 0; m < Run::kFloats / 4; ++m) {
+              const float4 f4 = run[m];
+              x[a][4 * m] = f4.x, x[a][4 * m + 1] = f4.y, x[a][4 * m + 2] = f4.z, x[a][4 * m + 3] = f4.w;
+            }
+          } else {
+            const float* run = lx + (tt * parts + part) * Run::kStride + (lane & 15);
+#pragma unroll
+            for (int m = 0; m < Run::kLoads; ++m) x[a][m] = run[16 * m];
           }
         }
 #pragma unroll
         for (int a = 0; a < kRows; ++a) {
           if (t0 + a < n) {
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int i = 0; i < KL; i += 4) {
-              const float qs[4] = {q4[a][i / 4].x, q4[a][i / 4].y, q4[a][i / 4].z, q4[a][i / 4].w};
-              const float ks[4] = {k4[a][i / 4].x, k4[a][i / 4].y, k4[a][i / 4].z, k4[a][i / 4].w};
-              const float ws[4] = {w4[a][i / 4].x, w4[a][i / 4].y, w4[a][i / 4].z, w4[a][i / 4].w};
-#pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const float kvv = ks[e] * vj[a];
-                if constexpr (kBefore) {
-                  acc[e] += qs[e] * (S[i + e] + u[i + e] * kvv);
-                  S[i + e] = ws[e] * S[i + e] + kvv;
-                } else {
-                  S[i + e] = ws[e] * S[i + e] + kvv;
-                  acc[e] += qs[e] * S[i + e];
-                }
+            static_for<0, KL>([&](auto at) {
+              constexpr int e = decltype(at)::value;
+              float qe, ke, we = head_decay;
+              if constexpr (kDirect) {
+                qe = x[a][e], ke = x[a][KL + e];
+                if constexpr (!kPerHead) we = x[a][2 * KL + e];
+              } else {
+                qe = row_lane<e % 16>(x[a][e / 16]), ke = row_lane<(KL + e) % 16>(x[a][(KL + e) / 16]);
+                if constexpr (!kPerHead) we = row_lane<(2 * KL + e) % 16>(x[a][(2 * KL + e) / 16]);
               }
-            }
-            lp[((t0 + a) * parts + wave * groups + group) * cw + col] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+              const float kvv = ke * vj[a];
+              if constexpr (kBefore) {
+                acc[e % 4] += qe * (S[e] + u[e] * kvv);
+                S[e] = we * S[e] + kvv;
+              } else {
+                S[e] = we * S[e] + kvv;
+                acc[e % 4] += qe * S[e];
+              }
+            });
+            lp[((t0 + a) * parts + part) * cw + col] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
           }
         }
       }
@@ -334,7 +367,7 @@ __global__ void __launch_bounds__(KL == 64 ? 512 : 256) linear_recurrence_kernel
       if (j0 + jj < dv) {
         float acc = 0.f;
         for (int g = 0; g < parts; ++g) acc += lp[(tt * parts + g) * cw + jj];
-        out[(static_cast<int64_t>(c0 + tt) * heads + head) * dv + j0 + jj] = acc;
+        out[kb * part_stride + (static_cast<int64_t>(c0 + tt) * heads + head) * dv + j0 + jj] = acc;
       }
     }
   }
@@ -402,34 +435,52 @@ extern "C" int alofa_shift_mix(void* out, const void* x, int dtype, const float*
 
 constexpr int kDecayApartFrom = 64;      // steps of more rows make their decays in a launch of their own
 
-// How a launch is shaped: the width of a block's slice of value channels (halved while a step has too few blocks to fill
-// the chip, down to 16), and from it the keys a lane keeps and the waves of a block (four where the key size allows).
+// How a launch is shaped. A step of few rows per request (decoding, short portions): a block owns all key channels of a head
+// and a slice of value channels, halved while the step has too few blocks to fill the chip, down to 16; from the slice's width
+// follow the keys a lane keeps and the waves of a block (four where the key size allows). A step of many rows (prompts), where
+// the caller has room for parts of the read-outs: slices of 64 value channels (a wave is one group, its operands come by
+// plain reads of one address), and the key channels of a head dealt out over blocks of 4 waves x 8 or 4 keys, so that a lone
+// prompt fills the chip with blocks that each issue few instructions a row.
 struct RecurrenceShape {
-  int cw_log2, kl, waves;
+  int cw_log2, kl, waves, key_blocks;
 };
-static inline RecurrenceShape recurrence_shape(int requests, int heads, int dk, int dv) {
+static inline RecurrenceShape recurrence_shape(int requests, int rows, int heads, int dk, int dv, int max_parts) {
   int cw_log2 = dv <= 16 ? 4 : dv <= 32 ? 5 : 6;
+  if (rows > kDecayApartFrom && max_parts > 1) {
+    const int groups = 64 >> cw_log2, slices = (dv + (1 << cw_log2) - 1) >> cw_log2;
+    for (int kl = 8; kl >= 4; kl /= 2) {
+      const int per_block = 4 * groups * kl, kb = (dk + per_block - 1) / per_block;
+      const bool fills = static_cast<int64_t>(requests) * heads * slices * kb >= compute_units();
+      if (kb <= max_parts && (fills || kl == 4 || 2 * kb > max_parts)) return {cw_log2, kl, 4, kb};
+    }
+  }
   const int64_t want = 2 * static_cast<int64_t>(compute_units());
   while (cw_log2 > 4 && static_cast<int64_t>(requests) * heads * ((dv + (1 << cw_log2) - 1) >> cw_log2) < want) --cw_log2;
   const int groups = 64 >> cw_log2;
   const int share = (dk + 4 * groups - 1) / (4 * groups);
   const int kl = share <= 4 ? 4 : share <= 8 ? 8 : share <= 16 ? 16 : share <= 32 ? 32 : 64;
-  return {cw_log2, kl, (dk + kl * groups - 1) / (kl * groups)};
+  return {cw_log2, kl, (dk + kl * groups - 1) / (kl * groups), 1};
 }
 
-static inline int recurrence_lds_bytes(const RecurrenceShape& s, int chunk) {
+static inline int recurrence_lds_bytes(const RecurrenceShape& s, int chunk, bool per_head) {
   const int groups = 64 >> s.cw_log2;
-  return chunk * (3 * s.waves * groups * s.kl + (1 << s.cw_log2) + s.waves * kWave) * static_cast<int>(sizeof(float));
+  const int loads = ((per_head ? 2 : 3) * s.kl + 15) / 16, stride = 16 * (loads | 1);      // (RunOfOperands)
+  return chunk * (s.waves * groups * stride + (1 << s.cw_log2) + s.waves * kWave) * static_cast<int>(sizeof(float));
 }
 
-extern "C" int alofa_linear_recurrence(float* out, const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
-                                       int dtype, float* decay_in, int64_t decay_stride, const float* decay_head, const float* bonus,
+// The most parts a step's read-outs may come in (the caller gives room for so many, or for one).
+extern "C" int alofa_linear_recurrence_max_parts(int dk) { return dk >= 32 ? min(8, (dk + 15) / 16) : 1; }
+
+// parts_used: in how many parts the read-outs were left (out + p * part_stride, p < parts_used; to be added by the reader).
+extern "C" int alofa_linear_recurrence(float* out, int max_parts, int64_t part_stride, int* parts_used, const void* q, int64_t q_stride, const void* k, int64_t k_stride,
+                                       const void* v, int64_t v_stride, int dtype, float* decay_in, int64_t decay_stride, const float* decay_head, const float* bonus,
                                        float* state, const int32_t* req_slot, const int32_t* row_off, int requests, int rows, int heads, int dk, int dv,
                                        int decay_kind, float tau, float q_scale, float k_scale, int before_update, hipStream_t stream) {
-  ALOFA_REQUIRE(requests >= 0 && heads > 0 && dk > 0 && dk <= 512 && dv > 0, "linear_recurrence: bad sizes (requests=%d heads=%d dk=%d dv=%d; dk at most 512)", requests, heads, dk, dv);
+  ALOFA_REQUIRE(requests >= 0 && heads > 0 && dk > 0 && dk <= 512 && dv > 0 && max_parts >= 1, "linear_recurrence: bad sizes (requests=%d heads=%d dk=%d dv=%d; dk at most 512)", requests, heads, dk, dv);
   ALOFA_REQUIRE(decay_kind >= kDecayPerHead && decay_kind <= kDecayGiven && rows >= requests, "linear_recurrence: no such kind of decay (%d), or fewer rows than requests", decay_kind);
   ALOFA_REQUIRE(decay_kind == kDecayPerHead ? decay_head != nullptr : decay_in != nullptr, "linear_recurrence: the decay's operand is absent");
   ALOFA_REQUIRE(decay_kind != kDecaySigmoidRoot || tau > 0.f, "linear_recurrence: tau must be positive");
+  *parts_used = 1;
   if (requests == 0) return 0;
   if (decay_kind != kDecayPerHead && decay_kind != kDecayGiven && rows > kDecayApartFrom) {
     const float inv = decay_kind == kDecaySigmoidRoot ? 1.f / tau : 0.f;
@@ -437,33 +488,47 @@ extern "C" int alofa_linear_recurrence(float* out, const void* q, int64_t q_stri
     if (check_launch("linear_recurrence (decays)")) return 1;
     decay_kind = kDecayGiven;
   }
-  const RecurrenceShape shape = recurrence_shape(requests, heads, dk, dv);
-  // rows staged in LDS at a time: sixteen, or as many as 64 KB hold for long keys; one where every request brings a single
-  // row (decoding: little LDS a block, so that many blocks share a compute unit and hide each other's waits)
-  int chunk = rows == requests ? 1 : 16;
+  const RecurrenceShape shape = recurrence_shape(requests, rows, heads, dk, dv, max_parts);
+  const bool per_head = decay_kind == kDecayPerHead;
+  // rows staged in LDS at a time: sixteen (thirty-two where a block has a share of the keys only), or as many as 64 KB hold for long
+  // keys; one where every request brings a single row (decoding: little LDS a block, so that many blocks share a compute unit
+  // and hide each other's waits)
+  int chunk = rows == requests ? 1 : shape.key_blocks > 1 ? 32 : 16;
   const int groups = 64 >> shape.cw_log2, threads = shape.waves * kWave;
   // (... and as a thread's registers fetch ahead: 16 values of q, k and the decay's operand each, 4 of v)
-  while (chunk > 1 && (recurrence_lds_bytes(shape, chunk) > 64 * 1024 || chunk * shape.waves * groups * shape.kl > 16 * threads || (chunk << shape.cw_log2) > 4 * threads)) chunk /= 2;
+  while (chunk > 1 && (recurrence_lds_bytes(shape, chunk, per_head) > 64 * 1024 || chunk * shape.waves * groups * shape.kl > 16 * threads || (chunk << shape.cw_log2) > 4 * threads)) chunk /= 2;
   ALOFA_REQUIRE(shape.waves * groups * shape.kl <= 16 * threads, "linear_recurrence: %d keys do not fit a block's registers", dk);
-  const int lds = recurrence_lds_bytes(shape, chunk);
-  ALOFA_REQUIRE(lds <= 64 * 1024 && shape.waves * kWave <= (shape.kl == 64 ? 512 : 256), "linear_recurrence: %d keys do not fit a block", dk);
+  const int lds = recurrence_lds_bytes(shape, chunk, per_head);
+  ALOFA_REQUIRE(lds <= 64 * 1024 && threads <= ((shape.kl <= 8 || shape.kl == 64) ? 512 : 256), "linear_recurrence: %d keys do not fit a block", dk);
   const int cw = 1 << shape.cw_log2;
-  const dim3 grid((dv + cw - 1) / cw, heads, requests), block(shape.waves * kWave);
+  const dim3 grid((dv + cw - 1) / cw, heads * shape.key_blocks, requests), block(threads);
   const float inv_tau = decay_kind == kDecaySigmoidRoot ? 1.f / tau : 0.f;
-#define ALOFA_SCAN(T, KL, PH) linear_recurrence_kernel<T, KL, PH><<<grid, block, lds, stream>>>(out, static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, \
-    static_cast<const T*>(v), v_stride, decay_in, decay_stride, decay_head, bonus, state, req_slot, row_off, heads, dk, dv, decay_kind, inv_tau, q_scale, k_scale, before_update, chunk, shape.cw_log2)
-#define ALOFA_SCAN_K(T, PH)                  \
-  switch (shape.kl) {                        \
-    case 4: ALOFA_SCAN(T, 4, PH); break;     \
-    case 8: ALOFA_SCAN(T, 8, PH); break;     \
-    case 16: ALOFA_SCAN(T, 16, PH); break;   \
-    case 32: ALOFA_SCAN(T, 32, PH); break;   \
-    default: ALOFA_SCAN(T, 64, PH); break;   \
+  *parts_used = shape.key_blocks;
+#define ALOFA_SCAN(T, KL, PH, DIRECT) linear_recurrence_kernel<T, KL, PH, DIRECT><<<grid, block, lds, stream>>>(out, static_cast<const T*>(q), q_stride, static_cast<const T*>(k), k_stride, \
+    static_cast<const T*>(v), v_stride, decay_in, decay_stride, decay_head, bonus, state, req_slot, row_off, heads, dk, dv, decay_kind, inv_tau, q_scale, k_scale, before_update, chunk, \
+    shape.cw_log2, shape.key_blocks, part_stride)
+#define ALOFA_SCAN_K(T, PH)                                                          \
+  if (groups == 1) {                                                                 \
+    switch (shape.kl) {                                                              \
+      case 4: ALOFA_SCAN(T, 4, PH, true); break;                                     \
+      case 8: ALOFA_SCAN(T, 8, PH, true); break;                                     \
+      case 16: ALOFA_SCAN(T, 16, PH, true); break;                                   \
+      case 32: ALOFA_SCAN(T, 32, PH, true); break;                                   \
+      default: ALOFA_SCAN(T, 64, PH, true); break;                                   \
+    }                                                                                \
+  } else {                                                                           \
+    switch (shape.kl) {                                                              \
+      case 4: ALOFA_SCAN(T, 4, PH, false); break;                                    \
+      case 8: ALOFA_SCAN(T, 8, PH, false); break;                                    \
+      case 16: ALOFA_SCAN(T, 16, PH, false); break;                                  \
+      case 32: ALOFA_SCAN(T, 32, PH, false); break;                                  \
+      default: ALOFA_SCAN(T, 64, PH, false); break;                                  \
+    }                                                                                \
   }
   if (dtype == kF32) {
-    if (decay_kind == kDecayPerHead) { ALOFA_SCAN_K(float, true) } else { ALOFA_SCAN_K(float, false) }
+    if (per_head) { ALOFA_SCAN_K(float, true) } else { ALOFA_SCAN_K(float, false) }
   } else {
-    if (decay_kind == kDecayPerHead) { ALOFA_SCAN_K(bf16_t, true) } else { ALOFA_SCAN_K(bf16_t, false) }
+    if (per_head) { ALOFA_SCAN_K(bf16_t, true) } else { ALOFA_SCAN_K(bf16_t, false) }
   }
 #undef ALOFA_SCAN_K
 #undef ALOFA_SCAN

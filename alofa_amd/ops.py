@@ -913,11 +913,19 @@ def layernorm(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, b: torch.Tens
 
 
 def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight: Optional[torch.Tensor], heads: int, dv: int,
-                  eps: float, exact: bool, out_scale: float = 1.0) -> None:
+                  eps: float, exact: bool, out_scale: float = 1.0, parts: int = 1) -> None:
     """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight[h, :] * silu(gate[t, h, :]); ``o`` float32
-    [T, heads * dv] contiguous, ``gate`` and ``out`` rows of heads * dv in the activation dtype (row strides allowed),
-    ``weight`` float32 [heads * dv] or None."""
-    _gpu("out", out, None, 2), _gpu("o", o, torch.float32, 2), _gpu("gate", gate, out.dtype, 2), _contig("o", o)
+    [T, heads * dv] contiguous, or [P, T, heads * dv] whose first ``parts`` are added first (read-outs that
+    ``linear_recurrence`` left in parts); ``gate`` and ``out`` rows of heads * dv in the activation dtype (row strides
+    allowed), ``weight`` float32 [heads * dv] or None."""
+    _gpu("out", out, None, 2), _gpu("o", o, torch.float32), _gpu("gate", gate, out.dtype, 2), _contig("o", o)
+    part_stride = 0
+    if o.dim() == 3:
+        if not 1 <= parts <= o.shape[0]:
+            raise AlofaError("shape_mismatch", "more parts than the read-outs have room for", f"o={tuple(o.shape)} parts={parts}")
+        part_stride, o = o.stride(0), o[0]
+    elif o.dim() != 2 or parts != 1:
+        raise AlofaError("shape_mismatch", "read-outs are [T, heads * dv] or parts of that", f"o={tuple(o.shape)} parts={parts}")
     T = o.shape[0]
     if o.shape[1] != heads * dv or tuple(out.shape) != (T, heads * dv) or tuple(gate.shape) != (T, heads * dv):
         raise AlofaError("shape_mismatch", "head norm operands do not fit", f"out={tuple(out.shape)} o={tuple(o.shape)} gate={tuple(gate.shape)} heads={heads} dv={dv}")
@@ -928,7 +936,7 @@ def headnorm_gate(out: torch.Tensor, o: torch.Tensor, gate: torch.Tensor, weight
     if exact and out.dtype is not torch.float32:
         raise AlofaError("invalid_argument", "the exact path is float32 throughout", f"out={out.dtype}")
     _call("alofa_headnorm_gate", _ptr(out), _L(_rows("out", out)), _ptr(o), _ptr(gate), _L(_rows("gate", gate)), _I(dtype_code(out)), _ptr(weight),
-          _I(T), _I(heads), _I(dv), _F(eps), _F(out_scale), _I(int(exact)), _stream())
+          _I(T), _I(heads), _I(dv), _F(eps), _F(out_scale), _I(parts), _L(part_stride), _I(int(exact)), _stream())
 
 
 XIELU, TANH = 0, 1
@@ -1069,19 +1077,29 @@ DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP, DECAY_GIVEN = 0, 1, 2, 3
 RECURRENCE_MAX_KEYS = 512
 
 
+def recurrence_max_parts(dk: int) -> int:
+    """In how many parts ``linear_recurrence`` may leave its read-outs when it is given room for them (``out`` [P, T, heads * dv])."""
+    return int(load().alofa_linear_recurrence_max_parts(_I(dk)))
+
+
 def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests,
                       heads: int, dk: int, dv: int, decay_kind: int, decay: torch.Tensor, tau: float = 1.0, bonus: Optional[torch.Tensor] = None,
-                      q_scale: float = 1.0, k_scale: float = 1.0, before_update: bool = False) -> None:
+                      q_scale: float = 1.0, k_scale: float = 1.0, before_update: bool = False) -> int:
     """Per request (in its rows' order) and head: S = diag(w_t) S + k_t v_t^T and out_t = S^T q_t, or with
     ``before_update`` out_t = (S + diag(bonus) k_t v_t^T)^T q_t first and the update after it. S float32
     [slots, heads, dk, dv] is read and left in ``state``. q, k [T, heads * dk] and v [T, heads * dv] are rows in one
-    dtype (row strides allowed); ``out`` float32 [T, heads * dv]. The decay w_t: ``DECAY_PER_HEAD`` with ``decay``
+    dtype (row strides allowed); ``out`` float32 [T, heads * dv], or [P, T, heads * dv]: then a step of many rows may deal a
+    head's key channels out over blocks, each of which leaves its part of the read-outs; the number of parts used is returned
+    (1 otherwise), and ``headnorm_gate(parts=)`` adds them. The decay w_t: ``DECAY_PER_HEAD`` with ``decay``
     float32 [heads]; ``DECAY_SIGMOID_ROOT`` sigmoid(z)^(1/tau) or ``DECAY_EXP_NEG_EXP`` exp(-exp(z)) with ``decay`` = z
     float32 [T, heads * dk] rows, which a step of many rows overwrites with the decays made of them; ``DECAY_GIVEN``:
     ``decay`` holds the w_t themselves."""
-    _gpu("out", out, torch.float32, 2), _contig("out", out), _gpu("q", q, None, 2), _gpu("k", k, q.dtype, 2), _gpu("v", v, q.dtype, 2)
+    _gpu("out", out, torch.float32), _contig("out", out), _gpu("q", q, None, 2), _gpu("k", k, q.dtype, 2), _gpu("v", v, q.dtype, 2)
     _gpu("state", state, torch.float32, 4), _contig("state", state)
     T = q.shape[0]
+    max_parts, part_stride = 1, 0
+    if out.dim() == 3:
+        max_parts, part_stride, out = out.shape[0], out.stride(0), out[0]
     if (tuple(q.shape) != (T, heads * dk) or tuple(k.shape) != (T, heads * dk) or tuple(v.shape) != (T, heads * dv) or tuple(out.shape) != (T, heads * dv)
             or tuple(state.shape[1:]) != (heads, dk, dv) or T != rows.rows or not 0 < dk <= RECURRENCE_MAX_KEYS):
         raise AlofaError("shape_mismatch", "recurrence operands do not fit", f"q={tuple(q.shape)} k={tuple(k.shape)} v={tuple(v.shape)} out={tuple(out.shape)} "
@@ -1097,7 +1115,9 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
         _gpu("bonus", bonus, torch.float32, 2), _contig("bonus", bonus)
         if tuple(bonus.shape) != (heads, dk) or not before_update:
             raise AlofaError("shape_mismatch", "the bonus is [heads, dk] and goes with the read-out before the update", f"bonus={tuple(bonus.shape)}")
-    _call("alofa_linear_recurrence", _ptr(out), _ptr(q), _L(_rows("q", q)), _ptr(k), _L(_rows("k", k)), _ptr(v), _L(_rows("v", v)), _I(dtype_code(q)),
+    used = _I(1)
+    _call("alofa_linear_recurrence", _ptr(out), _I(max_parts), _L(part_stride), ctypes.byref(used), _ptr(q), _L(_rows("q", q)), _ptr(k), _L(_rows("k", k)), _ptr(v), _L(_rows("v", v)), _I(dtype_code(q)),
           _ptr(None if per_head else decay), _L(0 if per_head else _rows("decay", decay)), _ptr(decay if per_head else None), _ptr(bonus), _ptr(state),
           _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(T), _I(heads), _I(dk), _I(dv), _I(decay_kind), _F(tau), _F(q_scale), _F(k_scale),
           _I(int(before_update)), _stream())
+    return used.value

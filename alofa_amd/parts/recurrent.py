@@ -48,10 +48,14 @@ class RecurrentMixer(Mixer):
     def state_need(self):
         return StateNeed((self.heads, self.dk, self.dv), torch.float32)
 
-    def _leave(self, ctx, o, gate, weight, residual, out):
-        """Head norm, gate and output projection of the read-outs ``o`` (float32 [T, heads * dv])."""
-        y = ctx.scratch("recurrent_gated", (o.shape[0], self.heads * self.dv), self.rt.dtype)
-        ops.headnorm_gate(y, o, gate, weight, self.heads, self.dv, self.eps, self.rt.exact)
+    def _readouts(self, ctx, rows: int):
+        """Room for the read-outs of a step: float32 [parts, T, heads * dv]; a step of many rows may leave them in parts."""
+        return ctx.scratch("recurrent_out", (ops.recurrence_max_parts(self.dk), rows, self.heads * self.dv), torch.float32)
+
+    def _leave(self, ctx, o, parts, gate, weight, residual, out):
+        """Head norm, gate and output projection of the read-outs ``o`` (float32 [P, T, heads * dv], the first ``parts`` to be added)."""
+        y = ctx.scratch("recurrent_gated", (o.shape[1], self.heads * self.dv), self.rt.dtype)
+        ops.headnorm_gate(y, o, gate, weight, self.heads, self.dv, self.eps, self.rt.exact, parts=parts)
         if out is not None:
             ops.gemm(out, y, self.w_o, exact=self.rt.exact)
         else:
@@ -101,10 +105,10 @@ class Retention(RecurrentMixer):
             self.position.apply(ctx, proj[:, :kd].unflatten(1, (self.heads, self.dk)), proj[:, kd:2 * kd].unflatten(1, (self.heads, self.dk)))
         else:      # queries and keys alike: 2 * heads heads to rotate, nothing to write to pages
             ops.rope_kv_write(proj, table[0], table[1], ctx.positions, 2 * self.heads, 0, self.dk)
-        o = ctx.scratch("recurrent_out", (T, vd), torch.float32)
-        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
-                              self.heads, self.dk, self.dv, ops.DECAY_PER_HEAD, self.decay, k_scale=self.k_scale)
-        self._leave(ctx, o, proj[:, 2 * kd + vd:], None, residual, out)
+        o = self._readouts(ctx, T)
+        parts = ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
+                                      self.heads, self.dk, self.dv, ops.DECAY_PER_HEAD, self.decay, k_scale=self.k_scale)
+        self._leave(ctx, o, parts, proj[:, 2 * kd + vd:], None, residual, out)
 
 
 class GatedLinearAttention(RecurrentMixer):
@@ -138,10 +142,10 @@ class GatedLinearAttention(RecurrentMixer):
         ops.gemm(proj, x, self.w_in, exact=self.rt.exact)
         z = ctx.scratch("recurrent_decay", (T, kd), torch.float32)
         ops.gemm(z, proj[:, 2 * kd + 2 * vd:], self.w_a2, self.b_a2, exact=self.rt.exact)
-        o = ctx.scratch("recurrent_out", (T, vd), torch.float32)
-        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
-                              self.heads, self.dk, self.dv, ops.DECAY_SIGMOID_ROOT, z, tau=self.tau, q_scale=self.q_scale)
-        self._leave(ctx, o, proj[:, 2 * kd + vd:2 * kd + 2 * vd], self.norm, residual, out)
+        o = self._readouts(ctx, T)
+        parts = ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:2 * kd + vd], ctx.state(where), rows_of_requests(ctx),
+                                      self.heads, self.dk, self.dv, ops.DECAY_SIGMOID_ROOT, z, tau=self.tau, q_scale=self.q_scale)
+        self._leave(ctx, o, parts, proj[:, 2 * kd + vd:2 * kd + 2 * vd], self.norm, residual, out)
 
 
 MIXES = ("r", "k", "v", "g", "w")
@@ -218,10 +222,10 @@ class TimeMix(RecurrentMixer):
         ops.activation(low, low, ops.TANH, exact=exact)
         z = ctx.scratch("recurrent_decay", (T, kd), torch.float32)
         ops.gemm(z, low, self.w["w2"], self.w0, exact=exact)
-        o = ctx.scratch("recurrent_out", (T, kd), torch.float32)
-        ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:3 * kd], ctx.state((entry, k)), rows_of_requests(ctx),
-                              self.heads, self.dk, self.dv, ops.DECAY_EXP_NEG_EXP, z, bonus=self.bonus, before_update=True)
-        self._leave(ctx, o, proj[:, 3 * kd:], self.norm, residual, out)
+        o = self._readouts(ctx, T)
+        parts = ops.linear_recurrence(o, proj[:, :kd], proj[:, kd:2 * kd], proj[:, 2 * kd:3 * kd], ctx.state((entry, k)), rows_of_requests(ctx),
+                                      self.heads, self.dk, self.dv, ops.DECAY_EXP_NEG_EXP, z, bonus=self.bonus, before_update=True)
+        self._leave(ctx, o, parts, proj[:, 3 * kd:], self.norm, residual, out)
 
 
 class ParallelMixers(Mixer):

@@ -146,10 +146,13 @@ def test_linear_recurrence(heads, dk, dv, kind, dtype):
         live = [(s, parts[s][step]) for s in (3, 0) if step < len(parts[s])]
         q, k, v, z = (np.concatenate([data[s][j][a:b] for s, (a, b) in live]) for j in range(4))
         rows = rows_of([(s, b - a) for s, (a, b) in live], n_slots)
-        out = torch.empty(q.shape[0], heads * dv, device=DEV)
+        # (room for the read-outs in parts: the step of 100 rows deals the key channels out over blocks where the key size allows)
+        room = torch.full((ops.recurrence_max_parts(dk), q.shape[0], heads * dv), float("nan"), device=DEV)
         decay = dev(per_head) if kind == "per_head" else dev(z - 2.0 if kind == "exp_neg_exp" else z)
-        ops.linear_recurrence(out, dev(q, dtype), dev(k, dtype), dev(v, dtype), state, rows, heads, dk, dv, code, decay, tau=tau,
-                              bonus=None if bonus is None else dev(bonus), q_scale=qs, k_scale=ks, before_update=bonus is not None)
+        used = ops.linear_recurrence(room, dev(q, dtype), dev(k, dtype), dev(v, dtype), state, rows, heads, dk, dv, code, decay, tau=tau,
+                                     bonus=None if bonus is None else dev(bonus), q_scale=qs, k_scale=ks, before_update=bonus is not None)
+        assert 1 <= used <= room.shape[0] and (used > 1) == (q.shape[0] > 64 and dk >= 32)
+        out = room[:used].sum(0)
         at = 0
         for s, (a, b) in live:
             got[s].append(out[at:at + b - a].cpu().numpy())
@@ -174,6 +177,11 @@ def test_head_norm_and_gate(heads, dv, weighted):
     out = torch.empty(T, heads * dv, device=DEV)
     ops.headnorm_gate(out, dev(o.reshape(T, -1)), wide[:, 8:], None if w is None else dev(w), heads, dv, 1e-6, True)
     assert np.abs(out.cpu().numpy() - want).max() <= 1e-5 * max(1.0, np.abs(want).max())
+    # the same read-outs in three parts, with room for four
+    shares = rng.normal(0, 1, (4, T, heads * dv)).astype(np.float32)
+    shares[2] = o.reshape(T, -1) - shares[0] - shares[1]
+    ops.headnorm_gate(out, dev(shares), wide[:, 8:], None if w is None else dev(w), heads, dv, 1e-6, True, parts=3)
+    assert np.abs(out.cpu().numpy() - want).max() <= 2e-5 * max(1.0, np.abs(want).max())
 
 
 def test_activations():
