@@ -511,13 +511,14 @@ def tugalix_sizes(width, heads, dim, ff, layers, vocab=32000):
     return tug, qwen
 
 
-DESIGN_SIZES = {"1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
+DESIGN_SIZES = {"256": (256, 4, 64, 1024, 4), "1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
+DESIGN_DEFAULT = ("1k", "2k", "4k")      # ("256": a small one, for a quick look)
 
 
 def designs(args):
     """Prefill (one prompt of 2,048 tokens in one step) and decode steps (batch 1, 8 and 64 at a context of about 550) of
     Tugalix beside Qwen2 at equal sizes, random weights: one line per point and model."""
-    sizes = [s for s in (args.sizes.split(",") if args.sizes else DESIGN_SIZES)]
+    sizes = args.sizes.split(",") if args.sizes else list(DESIGN_DEFAULT)
     for size in sizes:
         if size not in DESIGN_SIZES:
             print(f"no such size: {size} (known: {','.join(DESIGN_SIZES)})")
@@ -562,7 +563,7 @@ def main():
     ap.add_argument("--batches", default=None, help="with --sweep batch: these batch sizes only (comma-separated), e.g. to profile one point")
     ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
     ap.add_argument("--design", choices=["tugalix"], default=None, help="prefill and decode of this design beside Qwen2 at equal sizes (--sizes), a line per point")
-    ap.add_argument("--sizes", default=None, help=f"with --design: which of {','.join(DESIGN_SIZES)} (comma-separated; default all)")
+    ap.add_argument("--sizes", default=None, help=f"with --design: which of {','.join(DESIGN_SIZES)} (comma-separated; default {','.join(DESIGN_DEFAULT)})")
     ap.add_argument("--only", choices=["tugalix", "qwen2"], default=None, help="with --design: this model alone (for profiling)")
     ap.add_argument("--prompt-tokens", type=int, default=2048, help="with --design: tokens of the prefill point's prompt")
     ap.add_argument("--no-prefill", action="store_true", help="with --design: decode points only")

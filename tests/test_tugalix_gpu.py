@@ -206,3 +206,35 @@ def test_decode_steps_replay_a_captured_graph(replayers, tugalix_dirs):
     got = collect(r, bulk_and_tail("t", ids, tail=30))["t"]
     assert r.fn.graph_replays > before
     assert_close(got, plain_logits(tugalix_dirs[name], tuple(ids)), "bfloat16", "graph decode")
+
+
+def test_the_programs_take_the_design_by_its_config(tugalix_dirs, tmp_path):
+    """bin/generate and bin/trace_run on a folder whose config.json names the architecture plainly and leaves the ranks of
+    the decay projections to the tensors' shapes."""
+    import os
+    import subprocess
+    from conftest import ROOT
+    name = "A"
+    d = tmp_path / "bare"
+    d.mkdir()
+    raw = json.loads((tugalix_dirs[name] / "config.json").read_text())
+    del raw["layers"][1]["mixer"]["right"]["rank"], raw["layers"][2]["mixer"]["rank"]
+    (d / "config.json").write_text(json.dumps(raw))
+    (d / "model.safetensors").write_bytes((tugalix_dirs[name] / "model.safetensors").read_bytes())
+    cfg, w = plain_model(str(tugalix_dirs[name]))
+    prompts = [random_ids(1, 5, cfg["vocab"]), random_ids(2, 19, cfg["vocab"])]
+    want = [pt.greedy(w, cfg, p, 5) for p in prompts]
+    env = dict(os.environ, ALOFA_WEIGHTS=str(d), ALOFA_DTYPE="float32", ALOFA_MAX_NEW="5", ALOFA_MAX_TOKENS="64",
+               ALOFA_PROMPT_IDS=";".join(",".join(map(str, p)) for p in prompts))
+    p = subprocess.run([str(ROOT / "bin" / "generate")], env=env, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [[int(t) for t in line.split(",")] for line in p.stdout.strip().splitlines()] == want
+    ids = ids_of(name, seed=12, n=70)
+    steps = portions("a", ids, sizes=(33, 2, 1, 1, 20, 1))
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    p = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "bfloat16", "--out", str(tmp_path / "out"), "--max-tokens", "128"],
+                       input=text, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    got = np.concatenate([np.fromfile(tmp_path / "out" / f"{s['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab"]) for s in steps])
+    assert_close(got, plain_logits(tugalix_dirs[name], tuple(ids)), "bfloat16", "program")
