@@ -237,9 +237,9 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
 
   // A chunk's q, k and decay operands are fetched into registers while the chunk before runs (kFetch values of each per
   // thread), and go to LDS, decays made, once that one's read-outs are written.
-  constexpr int kFetch = 16;      // chunk * dk_pad <= kFetch * threads: the host sees to it
+  constexpr int kFetch = 16, kFetchV = 8;      // chunk * dk_pad <= kFetch * threads, chunk * cw <= kFetchV * threads: the host sees to it
   T fq[kFetch], fk[kFetch];
-  float fz[kFetch], fv[4];
+  float fz[kFetch], fv[kFetchV];
   // (value f of a thread is element threadIdx.x + f * threads of the chunk's [rows][dk_pad]: its row and channel follow from
   // the one before by additions, the only divisions are these)
   const int threads = blockDim.x;
@@ -263,7 +263,7 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
       }
     }
 #pragma unroll
-    for (int f = 0; f < 4; ++f) {
+    for (int f = 0; f < kFetchV; ++f) {
       if (f < v_passes) {
         const int e = threadIdx.x + f * threads;
         const int tv = e >> cw_log2, jj = e & (cw - 1);
@@ -301,7 +301,7 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
       }
     }
 #pragma unroll
-    for (int f = 0; f < 4; ++f) {
+    for (int f = 0; f < kFetchV; ++f) {
       const int e = threadIdx.x + f * threads;
       if (f < v_passes && e < n * cw) lv[e] = fv[f];
     }
@@ -311,26 +311,33 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
       constexpr bool kBefore = decltype(before)::value;
       // kRows rows at a time: their operands are asked of LDS together, then the rows run in order (a wave is alone on
       // its SIMD, so what it waits for is not hidden by others)
-      constexpr int kRows = kDirect ? (KL <= 8 ? 4 : KL == 16 ? 2 : 1) : (KL <= 16 ? 4 : KL == 32 ? 2 : 1);
-      for (int t0 = 0; t0 < n; t0 += kRows) {
-        float vj[kRows], x[kRows][kDirect ? Run::kFloats : Run::kLoads];
+      constexpr int kRows = kDirect ? (KL <= 4 ? 4 : KL <= 16 ? 2 : 1) : (KL <= 16 ? 4 : KL == 32 ? 2 : 1);
+      // ... and, in the shape of long steps, the next rows' operands are asked for before these rows run: two sets of registers take turns.
+      constexpr int kOperands = kDirect ? Run::kFloats : Run::kLoads;
+      const float* my_v = lv + col;
+      const float* my_run = lx + part * Run::kStride + (kDirect ? 0 : (lane & 15));
+      float* my_part = lp + part * cw + col;
+      const int run_step = parts * Run::kStride, part_step = parts * cw;
+      auto ask = [&](int t0, float (&vj)[kRows], float (&x)[kRows][kOperands]) {
 #pragma unroll
         for (int a = 0; a < kRows; ++a) {
-          const int tt = min(t0 + a, n - 1);
-          vj[a] = lv[tt * cw + col];
+          const int tt = min(t0 + a, n - 1);      // (rows past the chunk's end: read again, never used)
+          vj[a] = my_v[tt * cw];
           if constexpr (kDirect) {      // the wave is one group: every lane reads the whole run (reads of one address, 16 bytes at a time)
-            const float4* run = reinterpret_cast<const float4*>(lx + (tt * parts + part) * Run::kStride);
+            const float4* run = reinterpret_cast<const float4*>(my_run + tt * run_step);
 #pragma unroll
             for (int m = 0; m < Run::kFloats / 4; ++m) {
               const float4 f4 = run[m];
               x[a][4 * m] = f4.x, x[a][4 * m + 1] = f4.y, x[a][4 * m + 2] = f4.z, x[a][4 * m + 3] = f4.w;
             }
           } else {
-            const float* run = lx + (tt * parts + part) * Run::kStride + (lane & 15);
+            const float* run = my_run + tt * run_step;
 #pragma unroll
             for (int m = 0; m < Run::kLoads; ++m) x[a][m] = run[16 * m];
           }
         }
+      };
+      auto run = [&](int t0, const float (&vj)[kRows], const float (&x)[kRows][kOperands]) {
 #pragma unroll
         for (int a = 0; a < kRows; ++a) {
           if (t0 + a < n) {
@@ -354,8 +361,27 @@ __global__ void __launch_bounds__((KL <= 8 || KL == 64) ? 512 : 256) linear_recu
                 acc[e % 4] += qe * S[e];
               }
             });
-            lp[((t0 + a) * parts + part) * cw + col] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+            my_part[(t0 + a) * part_step] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
           }
+        }
+      };
+      float vj_a[kRows], x_a[kRows][kOperands];
+      if constexpr (kDirect && KL <= 8) {      // (the shape of long steps: few keys a lane)
+        float vj_b[kRows], x_b[kRows][kOperands];
+        ask(0, vj_a, x_a);
+        for (int t0 = 0; t0 < n; t0 += 2 * kRows) {
+          const bool more = t0 + kRows < n;
+          if (more) ask(t0 + kRows, vj_b, x_b);
+          run(t0, vj_a, x_a);
+          if (more) {
+            if (t0 + 2 * kRows < n) ask(t0 + 2 * kRows, vj_a, x_a);
+            run(t0 + kRows, vj_b, x_b);
+          }
+        }
+      } else {      // (steps of few rows: one set of registers, so that more blocks share a compute unit)
+        for (int t0 = 0; t0 < n; t0 += kRows) {
+          ask(t0, vj_a, x_a);
+          run(t0, vj_a, x_a);
         }
       }
     };
@@ -495,8 +521,8 @@ extern "C" int alofa_linear_recurrence(float* out, int max_parts, int64_t part_s
   // and hide each other's waits)
   int chunk = rows == requests ? 1 : shape.key_blocks > 1 ? 32 : 16;
   const int groups = 64 >> shape.cw_log2, threads = shape.waves * kWave;
-  // (... and as a thread's registers fetch ahead: 16 values of q, k and the decay's operand each, 4 of v)
-  while (chunk > 1 && (recurrence_lds_bytes(shape, chunk, per_head) > 64 * 1024 || chunk * shape.waves * groups * shape.kl > 16 * threads || (chunk << shape.cw_log2) > 4 * threads)) chunk /= 2;
+  // (... and as a thread's registers fetch ahead: 16 values of q, k and the decay's operand each, 8 of v)
+  while (chunk > 1 && (recurrence_lds_bytes(shape, chunk, per_head) > 64 * 1024 || chunk * shape.waves * groups * shape.kl > 16 * threads || (chunk << shape.cw_log2) > 8 * threads)) chunk /= 2;
   ALOFA_REQUIRE(shape.waves * groups * shape.kl <= 16 * threads, "linear_recurrence: %d keys do not fit a block's registers", dk);
   const int lds = recurrence_lds_bytes(shape, chunk, per_head);
   ALOFA_REQUIRE(lds <= 64 * 1024 && threads <= ((shape.kl <= 8 || shape.kl == 64) ? 512 : 256), "linear_recurrence: %d keys do not fit a block", dk);
