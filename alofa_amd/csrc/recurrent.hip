@@ -117,20 +117,23 @@ __global__ void __launch_bounds__(256) norm_conv_step_kernel(TO* __restrict__ ou
 
 // ---- mix with the token before --------------------------------------------------------------------------
 // out[s, t, c] = x[t, c] + (x[t-1, c] - x[t, c]) * mu[s, c] for s < n_mixes; the row before a request's first row
-// of this step is state[slot, c] (zeros for a new request). The state is kept by keep_last_rows (keep = 1).
+// of this step is state[slot, c] (zeros for a new request). The state is kept by keep_last_rows (keep = 1), or, in steps of
+// single rows (row_off absent) with `keep` set, here: the thread that read a request's channel writes the row over it.
 template <typename T>
 __global__ void __launch_bounds__(256) shift_mix_kernel(T* __restrict__ out, const T* __restrict__ x, const float* __restrict__ mu,
-                                                        const T* __restrict__ state, const int32_t* __restrict__ req_slot,
+                                                        T* __restrict__ state, const int32_t* __restrict__ req_slot,
                                                         const int32_t* __restrict__ row_off, const int32_t* __restrict__ req_of_row,
-                                                        int rows, int width, int n_mixes) {
+                                                        int rows, int width, int n_mixes, int keep) {
   const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (idx >= static_cast<int64_t>(rows) * width) return;
   const int t = static_cast<int>(idx / width), c = static_cast<int>(idx % width);
   const int r = req_of_row ? req_of_row[t] : t;
   const int row0 = row_off ? row_off[r] : r;
-  const float cur = load_f32(x + static_cast<int64_t>(t) * width + c);
-  const float prev = t > row0 ? load_f32(x + static_cast<int64_t>(t - 1) * width + c)
-                              : load_f32(state + static_cast<int64_t>(req_slot[r]) * width + c);
+  const T mine = x[static_cast<int64_t>(t) * width + c];
+  const float cur = load_f32(&mine);
+  T* kept = state + static_cast<int64_t>(req_slot[r]) * width + c;
+  const float prev = t > row0 ? load_f32(x + static_cast<int64_t>(t - 1) * width + c) : load_f32(kept);
+  if (keep) *kept = mine;
   const float diff = prev - cur;
   for (int s = 0; s < n_mixes; ++s)
     store_f32(out + (static_cast<int64_t>(s) * rows + t) * width + c, cur + diff * mu[static_cast<int64_t>(s) * width + c]);
@@ -449,13 +452,14 @@ extern "C" int alofa_keep_last_rows(void* state, const void* h, int dtype, const
   return check_launch("keep_last_rows");
 }
 
-extern "C" int alofa_shift_mix(void* out, const void* x, int dtype, const float* mu, const void* state, const int32_t* req_slot, const int32_t* row_off,
-                               const int32_t* req_of_row, int rows, int width, int n_mixes, hipStream_t stream) {
+extern "C" int alofa_shift_mix(void* out, const void* x, int dtype, const float* mu, void* state, const int32_t* req_slot, const int32_t* row_off,
+                               const int32_t* req_of_row, int rows, int width, int n_mixes, int keep, hipStream_t stream) {
   ALOFA_REQUIRE(rows >= 0 && width > 0 && n_mixes >= 1, "shift_mix: bad sizes (rows=%d width=%d mixes=%d)", rows, width, n_mixes);
+  ALOFA_REQUIRE(!keep || row_off == nullptr, "shift_mix: the state is kept here only in steps of single rows");
   if (rows == 0) return 0;
   const unsigned grid = blocks_of(static_cast<int64_t>(rows) * width);
-  if (dtype == kF32) shift_mix_kernel<float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), static_cast<const float*>(x), mu, static_cast<const float*>(state), req_slot, row_off, req_of_row, rows, width, n_mixes);
-  else shift_mix_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(x), mu, static_cast<const bf16_t*>(state), req_slot, row_off, req_of_row, rows, width, n_mixes);
+  if (dtype == kF32) shift_mix_kernel<float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), static_cast<const float*>(x), mu, static_cast<float*>(state), req_slot, row_off, req_of_row, rows, width, n_mixes, keep);
+  else shift_mix_kernel<bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), static_cast<const bf16_t*>(x), mu, static_cast<bf16_t*>(state), req_slot, row_off, req_of_row, rows, width, n_mixes, keep);
   return check_launch("shift_mix");
 }
 

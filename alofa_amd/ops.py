@@ -1060,17 +1060,20 @@ def keep_last_rows(state: torch.Tensor, h: torch.Tensor, rows: RowsOfRequests) -
           _I(state.shape[1]), _stream())
 
 
-def shift_mix(out: torch.Tensor, x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests) -> None:
+def shift_mix(out: torch.Tensor, x: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests, keep: bool = False) -> None:
     """out[s, t] = x[t] + (x[t - 1] - x[t]) * mu[s], the row before a request's first row of this step taken from
-    ``state`` [slots, 1, width] (x's dtype; not written). ``mu`` float32 [n, width]; out [n, T, width] in x's dtype."""
+    ``state`` [slots, 1, width] (x's dtype). ``mu`` float32 [n, width]; out [n, T, width] in x's dtype. The state is not
+    written (``keep_last_rows`` does that), unless ``keep`` is set in a step of single rows: then it moves on in the same launch."""
     _gpu("out", out, x.dtype, 3), _gpu("x", x, None, 2), _gpu("mu", mu, torch.float32, 2), _gpu("state", state, x.dtype, 3)
     _contig("out", out), _contig("x", x), _contig("mu", mu), _contig("state", state)
     T, width = x.shape
     if tuple(out.shape) != (mu.shape[0], T, width) or mu.shape[1] != width or tuple(state.shape[1:]) != (1, width) or T != rows.rows:
         raise AlofaError("shape_mismatch", "token mix operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} mu={tuple(mu.shape)} state={tuple(state.shape)}")
     rows.fits("state", state)
+    if keep and rows.offsets is not None:
+        raise AlofaError("invalid_argument", "the token mix keeps its state itself only in steps of single rows")
     _call("alofa_shift_mix", _ptr(out), _ptr(x), _I(dtype_code(x)), _ptr(mu), _ptr(state), _ptr(rows.slots), _ptr(rows.offsets), _ptr(rows.req_of_row),
-          _I(T), _I(width), _I(mu.shape[0]), _stream())
+          _I(T), _I(width), _I(mu.shape[0]), _I(int(keep)), _stream())
 
 
 DECAY_PER_HEAD, DECAY_SIGMOID_ROOT, DECAY_EXP_NEG_EXP, DECAY_GIVEN = 0, 1, 2, 3

@@ -170,8 +170,10 @@ class TokenShift(TimeConv):
 
     def forward(self, ctx, where, out, x):
         state, rows = ctx.state(where), rows_of_requests(ctx)
-        ops.shift_mix(out, x, self.mu, state, rows)
-        ops.keep_last_rows(state, x, rows)
+        single = rows.offsets is None      # single rows (decoding): the mix and the state's step are one launch
+        ops.shift_mix(out, x, self.mu, state, rows, keep=single)
+        if not single:
+            ops.keep_last_rows(state, x, rows)
 
 
 class TimeMix(RecurrentMixer):

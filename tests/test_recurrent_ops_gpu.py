@@ -96,11 +96,14 @@ def test_mix_with_the_token_before():
     want = np.stack([x + (before - x) * m for m in mu])
     state = torch.zeros(3, 1, width, device=DEV)
     got = []
-    for a, b in cuts(11, (1, 1, 4, 2, 3)):
+    for a, b in cuts(11, (1, 1, 4, 2, 1, 1, 1)):
         rows = rows_of([(2, b - a)], 3)
         out = torch.empty(5, b - a, width, device=DEV)
-        ops.shift_mix(out, dev(x[a:b]), dev(mu), state, rows)
-        ops.keep_last_rows(state, dev(x[a:b]), rows)
+        if b - a == 1 and a % 2:      # a single row: the state may move on in the same launch
+            ops.shift_mix(out, dev(x[a:b]), dev(mu), state, rows, keep=True)
+        else:
+            ops.shift_mix(out, dev(x[a:b]), dev(mu), state, rows)
+            ops.keep_last_rows(state, dev(x[a:b]), rows)
         got.append(out.cpu().numpy())
     assert np.abs(np.concatenate(got, axis=1) - want).max() <= 1e-6
 
