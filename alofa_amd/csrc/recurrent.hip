@@ -47,7 +47,7 @@ __global__ void __launch_bounds__(256) short_conv_kernel(TO* __restrict__ out, c
 // The last `keep` rows a request has seen, after this step: state[slot, i, c] = the input at (end of the request's
 // rows) - keep + i, from this step's rows or, where the step brought fewer, from the old state. A thread owns one
 // channel of one request, reads what it needs and writes afterwards.
-constexpr int kMaxKeep = 8;
+constexpr int kMaxKeep = 15;
 template <typename TI>
 __global__ void __launch_bounds__(256) keep_last_rows_kernel(TI* __restrict__ state, const TI* __restrict__ h, const int32_t* __restrict__ req_slot,
                                                              const int32_t* __restrict__ row_off, int requests, int width, int keep) {

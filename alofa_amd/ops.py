@@ -1009,7 +1009,7 @@ class RowsOfRequests:
             raise AlofaError("shape_mismatch", "the state has fewer slots than the step's requests may name", f"operand={name} state={tuple(state.shape)} slots={self.n_slots}")
 
 
-CONV_MAX_TAPS = 9
+CONV_MAX_TAPS = 16
 
 
 def short_conv(out: torch.Tensor, h: torch.Tensor, w: torch.Tensor, state: torch.Tensor, rows: RowsOfRequests, exact: bool = False) -> None:

@@ -55,7 +55,7 @@ def test_layer_norm(width, exact):
     assert torch.equal(inplace, out)
 
 
-@pytest.mark.parametrize("taps", [1, 2, 3, 4, 9])
+@pytest.mark.parametrize("taps", [1, 2, 3, 4, 9, 16])
 def test_short_convolution_in_portions_of_two_requests(taps):
     """Two requests whose rows arrive in unequal portions within the same calls; the state carries the last rows."""
     from alofa_amd import ops
@@ -244,7 +244,7 @@ def test_part_of_a_head_rotated():
     assert np.abs(np.einsum("thd,shd->hts", got[:, 0], got[:, 1]) - want).max() <= 1e-4
 
 
-@pytest.mark.parametrize("taps", [2, 4])
+@pytest.mark.parametrize("taps", [2, 4, 16])
 @pytest.mark.parametrize("exact", [True, False])
 def test_norm_filter_and_state_in_one_launch(taps, exact):
     """Single rows of three requests: the fused kernel against norm, filter and state update one after the other."""
