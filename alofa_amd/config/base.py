@@ -45,9 +45,12 @@ class LayerSpec:
 class RunEntry:
     """One entry of the run order. ``layer`` indexes ``ModelSpec.layers`` (a
     layer may be named twice). ``cache_of`` is None when the entry keeps a
-    cache of its own, else the index of the earlier entry whose cache it reads."""
+    cache of its own, else the index of the earlier entry whose cache it reads.
+    ``join``: None, or the index into ``ModelSpec.joins`` of the part that is applied to the stream
+    (beside the embedding's output) right before this entry runs."""
     layer: int
     cache_of: Optional[int] = None
+    join: Optional[int] = None
 
 
 @dataclass(frozen=True)
@@ -60,6 +63,7 @@ class ModelSpec:
     order: tuple             # RunEntry
     final_norm: PartSpec
     head: PartSpec
+    joins: tuple = ()        # PartSpec of the "join" family: what run entries name with ``join``
 
 
 class ModelConfig:

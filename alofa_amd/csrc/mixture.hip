@@ -1,0 +1,107 @@
+// Feed-forwards of which every token takes a few (a mixture of experts): the choice, and the gated
+// activation of the experts.
+//
+// The choice is float arithmetic on float scores (double in the exact path); ties go to the lower index.
+#include "common.h"
+
+namespace alofa {
+
+// ---- the choice -------------------------------------------------------------------------------
+// z [T, E] router products. Per token the `top` experts with the largest z (the same as the largest
+// sigmoid(z), without its saturation), the lower index first among equals. Outputs:
+//   dense [T, E]: sigmoid(z) * scale at the chosen experts, 0 elsewhere (weights sum to one first when `renorm`);
+//   chosen [T, top], weights [T, top]: the same as lists, in order of falling score.
+// One thread per token; E up to kMaxExperts.
+constexpr int kMaxExperts = 512;
+
+template <typename Acc>
+__global__ void __launch_bounds__(64) route_top_kernel(const float* __restrict__ z, float* __restrict__ dense, int32_t* __restrict__ chosen,
+                                                       float* __restrict__ weights, int tokens, int experts, int top, float scale, int renorm) {
+  const int t = blockIdx.x * 64 + threadIdx.x;
+  if (t >= tokens) return;
+  const float* row = z + static_cast<int64_t>(t) * experts;
+  float* d = dense + static_cast<int64_t>(t) * experts;
+  for (int e = 0; e < experts; ++e) d[e] = 0.f;
+  Acc total = 0;
+  float last = 0.f;
+  int last_e = -1;
+  for (int k = 0; k < top; ++k) {
+    // the largest score below (last, last_e) in the order (score falling, index rising)
+    int best = -1;
+    float best_z = 0.f;
+    for (int e = 0; e < experts; ++e) {
+      const float v = row[e];
+      const bool after = k == 0 || v < last || (v == last && e > last_e);
+      if (after && (best < 0 || v > best_z)) {
+        best = e;
+        best_z = v;
+      }
+    }
+    last = best_z;
+    last_e = best;
+    const Acc s = static_cast<Acc>(1) / (static_cast<Acc>(1) + exp(-static_cast<Acc>(best_z)));
+    total += s;
+    chosen[static_cast<int64_t>(t) * top + k] = best;
+    weights[static_cast<int64_t>(t) * top + k] = static_cast<float>(s);
+  }
+  for (int k = 0; k < top; ++k) {
+    Acc w = static_cast<Acc>(weights[static_cast<int64_t>(t) * top + k]);
+    if (renorm) w /= total;
+    const float f = static_cast<float>(w * static_cast<Acc>(scale));
+    weights[static_cast<int64_t>(t) * top + k] = f;
+    d[chosen[static_cast<int64_t>(t) * top + k]] = f;
+  }
+}
+
+// ---- gated activation of all experts side by side ------------------------------------------------
+// g, u [T, F]: gate and up products of every expert (E experts of `ff` channels each, then `shared_ff` channels of an
+// expert every token takes). act[t, c] = w * a * sigmoid(slope * a) * (b + 1) with a = min(g, limit),
+// b = clamp(u, -limit, limit), and w = dense[t, expert of c] (0: the token does not take that expert) or 1 for the
+// shared channels.
+template <typename T, typename Acc>
+__global__ void __launch_bounds__(256) clamped_glu_kernel(T* __restrict__ act, const T* __restrict__ g, const T* __restrict__ u, const float* __restrict__ dense,
+                                                          int64_t rows, int experts, int ff, int shared_ff, float limit, float shared_limit, float slope) {
+  const int F = experts * ff + shared_ff;
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * F) return;
+  const int64_t t = idx / F;
+  const int c = static_cast<int>(idx % F);
+  const bool own = c < experts * ff;
+  const float w = own ? dense[t * experts + c / ff] : 1.f;
+  float y = 0.f;
+  if (w != 0.f) {
+    const Acc lim = static_cast<Acc>(own ? limit : shared_limit);
+    Acc a = static_cast<Acc>(load_f32(g + idx)), b = static_cast<Acc>(load_f32(u + idx));
+    a = a < lim ? a : lim;
+    b = b < -lim ? -lim : (b > lim ? lim : b);
+    const Acc s = static_cast<Acc>(1) / (static_cast<Acc>(1) + exp(-static_cast<Acc>(slope) * a));
+    y = static_cast<float>(static_cast<Acc>(w) * (a * s * (b + static_cast<Acc>(1))));
+  }
+  store_f32(act + idx, y);
+}
+
+}  // namespace alofa
+
+using namespace alofa;
+
+extern "C" int alofa_route_top(const float* z, float* dense, int32_t* chosen, float* weights, int tokens, int experts, int top, float scale, int renorm,
+                               int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens >= 0 && experts > 0 && experts <= kMaxExperts && top > 0 && top <= experts, "route_top: bad sizes (tokens=%d experts=%d top=%d)", tokens, experts, top);
+  if (tokens == 0) return 0;
+  const unsigned grid = static_cast<unsigned>((tokens + 63) / 64);
+  if (exact) route_top_kernel<double><<<grid, 64, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
+  else route_top_kernel<float><<<grid, 64, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
+  return check_launch("route_top");
+}
+
+extern "C" int alofa_clamped_glu(void* act, const void* g, const void* u, int dtype, const float* dense, int64_t rows, int experts, int ff, int shared_ff,
+                                 float limit, float shared_limit, float slope, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && experts >= 0 && ff >= 0 && shared_ff >= 0 && experts * ff + shared_ff > 0 && (experts == 0 || dense), "clamped_glu: bad sizes");
+  ALOFA_REQUIRE(!exact || dtype == kF32, "clamped_glu: the exact path is float32");
+  if (rows == 0) return 0;
+  const unsigned grid = static_cast<unsigned>((rows * (experts * ff + shared_ff) + 255) / 256);
+  if (exact) clamped_glu_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(act), static_cast<const float*>(g), static_cast<const float*>(u), dense, rows, experts, ff, shared_ff, limit, shared_limit, slope);
+  else if (dtype == kF32) clamped_glu_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(act), static_cast<const float*>(g), static_cast<const float*>(u), dense, rows, experts, ff, shared_ff, limit, shared_limit, slope);
+  else clamped_glu_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(act), static_cast<const bf16_t*>(g), static_cast<const bf16_t*>(u), dense, rows, experts, ff, shared_ff, limit, shared_limit, slope);
+  return check_launch("clamped_glu");
+}

@@ -207,3 +207,205 @@ extern "C" int alofa_scale(float* x, float s, int64_t elements, hipStream_t stre
   scale_kernel<<<blocks_of(elements), 256, 0, stream>>>(x, s, elements);
   return check_launch("scale");
 }
+
+// =================================================================================================
+// Kernels of designs whose sub-layers are scaled channel by channel on their way into the stream,
+// whose embedding adds a row named by a hash of two tokens, and whose stream is joined with the
+// embedding's output by a projection.
+namespace alofa {
+
+// ---- token row times a factor, plus the row of a second table named by (token before, token) ----------
+// out[t] = table[id] * scale + pairs[(before * mul_prev + id * mul_cur) mod buckets]; for a request's first token
+// (position 0) the row `buckets`. The token before row t is row t - 1's within a request's rows, and for the first
+// row of a request in this step what `state` holds for its slot. The block of a request's first row then leaves the
+// request's last token of this step there (it alone touches the slot: read, barrier, write). Negative ids name tokens
+// in `store`, as in embed_gather.
+__device__ __forceinline__ int token_at(const int32_t* ids, int t, const int32_t* store, int vocab) {
+  int id = ids[t];
+  if (id < 0) {
+    id = store[-(id + 1)];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  }
+  return id;
+}
+
+template <typename TW>
+__global__ void pair_embed_kernel(float* __restrict__ out, const TW* __restrict__ table, const TW* __restrict__ pairs,
+                                  const int32_t* __restrict__ ids, const int32_t* __restrict__ positions, int32_t* state,
+                                  const int32_t* __restrict__ req_slot, const int32_t* __restrict__ row_off, const int32_t* __restrict__ req_of_row,
+                                  int width, const int32_t* __restrict__ store, int vocab, float scale,
+                                  int64_t buckets, int64_t mul_prev, int64_t mul_cur) {
+  const int t = blockIdx.x;
+  int first = t, last = t, slot = 0;
+  if (pairs) {
+    const int r = req_of_row ? req_of_row[t] : t;
+    if (row_off) first = row_off[r], last = row_off[r + 1] - 1;
+    slot = req_slot[r];
+  }
+  const int id = token_at(ids, t, store, vocab);
+  int64_t row = buckets;
+  if (pairs && positions[t] != 0) {
+    const int64_t before = t == first ? state[slot] : token_at(ids, t - 1, store, vocab);
+    row = (before * mul_prev + static_cast<int64_t>(id) * mul_cur) % buckets;
+    if (row < 0) row += buckets;
+  }
+  const TW* a = table + static_cast<int64_t>(id) * width;
+  float* dst = out + static_cast<int64_t>(t) * width;
+  if (pairs) {
+    const TW* b = pairs + row * width;
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_f32(a + c) * scale + load_f32(b + c);
+  } else {
+    for (int c = threadIdx.x; c < width; c += blockDim.x) dst[c] = load_f32(a + c) * scale;
+  }
+  if (state && t == first) {
+    const int keep = token_at(ids, last, store, vocab);
+    __syncthreads();
+    if (threadIdx.x == 0) state[slot] = keep;
+  }
+}
+
+// ---- out[t] = [a[t] | b[t]] in the activation type (two float streams side by side, the operand of one product) ----
+template <typename TO>
+__global__ void __launch_bounds__(256) concat_rows_kernel(TO* __restrict__ out, const float* __restrict__ a, const float* __restrict__ b, int64_t rows, int width) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * 2 * width) return;
+  const int64_t r = idx / (2 * width);
+  const int c = static_cast<int>(idx % (2 * width));
+  store_f32(out + idx, c < width ? a[r * width + c] : b[r * width + c - width]);
+}
+
+// ---- RMSNorm of short rows, left several times side by side ------------------------------------------------
+// y = x / sqrt(mean(x^2) + eps) * w of `width` values; out[t, k * pad + j] = y[j] for k < copies, zeros for
+// width <= j < pad. One wavefront per row.
+template <typename TO, typename Acc>
+__global__ void __launch_bounds__(256) rmsnorm_spread_kernel(TO* __restrict__ out, int64_t out_stride, const float* __restrict__ x, int64_t x_stride,
+                                                             const float* __restrict__ w, int rows, int width, int pad, int copies, float eps) {
+  const int t = blockIdx.x * 4 + threadIdx.x / kWave;
+  if (t >= rows) return;
+  const int lane = threadIdx.x % kWave;
+  const float* src = x + static_cast<int64_t>(t) * x_stride;
+  Acc ss = 0;
+  for (int j = lane; j < width; j += kWave) ss += static_cast<Acc>(src[j]) * static_cast<Acc>(src[j]);
+  ss = wave_sum(ss);
+  const Acc inv = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(width) + static_cast<Acc>(eps));
+  TO* dst = out + static_cast<int64_t>(t) * out_stride;
+  for (int j = lane; j < pad; j += kWave) {
+    const float y = j < width ? static_cast<float>(static_cast<Acc>(src[j]) * inv * static_cast<Acc>(w[j])) : 0.f;
+    for (int k = 0; k < copies; ++k) store_f32(dst + static_cast<int64_t>(k) * pad + j, y);
+  }
+}
+
+// ---- x[t, c] *= sigmoid(g[t, c]) ------------------------------------------------------------------------------
+template <typename T, typename Acc>
+__global__ void __launch_bounds__(256) sigmoid_gate_kernel(T* __restrict__ x, int64_t x_stride, const T* __restrict__ g, int64_t g_stride, int64_t rows, int width) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * width) return;
+  const int64_t r = idx / width;
+  const int c = static_cast<int>(idx % width);
+  const Acc z = static_cast<Acc>(load_f32(g + r * g_stride + c));
+  const Acc s = static_cast<Acc>(1) / (static_cast<Acc>(1) + exp(-z));
+  store_f32(x + r * x_stride + c, static_cast<float>(static_cast<Acc>(load_f32(x + r * x_stride + c)) * s));
+}
+
+// ---- residual[t, c] += scale[c] * x[t, c] ------------------------------------------------------------------------
+template <typename Acc>
+__global__ void __launch_bounds__(256) add_channel_scaled_kernel(float* __restrict__ residual, const float* __restrict__ x, const float* __restrict__ scale,
+                                                                 int64_t elements, int width) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e >= elements) return;
+  residual[e] = static_cast<float>(static_cast<Acc>(residual[e]) + static_cast<Acc>(scale[e % width]) * static_cast<Acc>(x[e]));
+}
+
+// ---- x = cap * tanh(x / cap) ---------------------------------------------------------------------------------------
+template <typename Acc>
+__global__ void __launch_bounds__(256) softcap_kernel(float* __restrict__ x, float cap, int64_t elements) {
+  const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (e < elements) x[e] = static_cast<float>(static_cast<Acc>(cap) * tanh(static_cast<Acc>(x[e]) / static_cast<Acc>(cap)));
+}
+
+// ---- the square of relu --------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) relu_squared_kernel(T* __restrict__ out, int64_t out_stride, const T* __restrict__ x, int64_t x_stride, int64_t rows, int width) {
+  const int64_t idx = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (idx >= rows * width) return;
+  const int64_t r = idx / width;
+  const int c = static_cast<int>(idx % width);
+  const float z = fmaxf(load_f32(x + r * x_stride + c), 0.f);
+  store_f32(out + r * out_stride + c, z * z);
+}
+
+}  // namespace alofa
+
+extern "C" int alofa_pair_embed(float* out, const void* table, const void* pairs, int table_dtype, const int32_t* ids, const int32_t* positions, int32_t* state,
+                                const int32_t* req_slot, const int32_t* row_off, const int32_t* req_of_row, int tokens, int width, const int32_t* store,
+                                int vocab, float scale, int64_t buckets, int64_t mul_prev, int64_t mul_cur, hipStream_t stream) {
+  ALOFA_REQUIRE(tokens > 0 && width > 0 && vocab > 0, "pair_embed: tokens=%d width=%d vocab=%d must be positive", tokens, width, vocab);
+  ALOFA_REQUIRE(pairs == nullptr || (buckets > 0 && state && positions && req_slot), "pair_embed: a pair table comes with buckets, positions, slots and state");
+  ALOFA_REQUIRE((row_off == nullptr) == (req_of_row == nullptr), "pair_embed: row offsets and request indices come together");
+  const int threads = width >= 256 ? 256 : 64;
+  if (table_dtype == kF32)
+    pair_embed_kernel<float><<<tokens, threads, 0, stream>>>(out, static_cast<const float*>(table), static_cast<const float*>(pairs), ids, positions, pairs ? state : nullptr,
+                                                             req_slot, row_off, req_of_row, width, store, vocab, scale, buckets, mul_prev, mul_cur);
+  else if (table_dtype == kBF16)
+    pair_embed_kernel<bf16_t><<<tokens, threads, 0, stream>>>(out, static_cast<const bf16_t*>(table), static_cast<const bf16_t*>(pairs), ids, positions, pairs ? state : nullptr,
+                                                              req_slot, row_off, req_of_row, width, store, vocab, scale, buckets, mul_prev, mul_cur);
+  else
+    ALOFA_REQUIRE(false, "pair_embed: unknown table dtype %d", table_dtype);
+  return check_launch("pair_embed");
+}
+
+extern "C" int alofa_concat_rows(void* out, int out_dtype, const float* a, const float* b, int64_t rows, int width, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0, "concat_rows: bad sizes");
+  if (rows == 0) return 0;
+  if (out_dtype == kF32) concat_rows_kernel<float><<<blocks_of(rows * 2 * width), 256, 0, stream>>>(static_cast<float*>(out), a, b, rows, width);
+  else concat_rows_kernel<bf16_t><<<blocks_of(rows * 2 * width), 256, 0, stream>>>(static_cast<bf16_t*>(out), a, b, rows, width);
+  return check_launch("concat_rows");
+}
+
+extern "C" int alofa_rmsnorm_spread(void* out, int out_dtype, int64_t out_stride, const float* x, int64_t x_stride, const float* w, int rows, int width, int pad,
+                                    int copies, float eps, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && pad >= width && copies >= 1 && eps > 0.f && out_stride >= static_cast<int64_t>(copies) * pad && x_stride >= width,
+                "rmsnorm_spread: bad sizes (rows=%d width=%d pad=%d copies=%d)", rows, width, pad, copies);
+  ALOFA_REQUIRE(!exact || out_dtype == kF32, "rmsnorm_spread: the exact path writes float32");
+  if (rows == 0) return 0;
+  const unsigned grid = static_cast<unsigned>((rows + 3) / 4);
+  if (exact) rmsnorm_spread_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
+  else if (out_dtype == kF32) rmsnorm_spread_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
+  else rmsnorm_spread_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
+  return check_launch("rmsnorm_spread");
+}
+
+extern "C" int alofa_sigmoid_gate(void* x, int64_t x_stride, const void* g, int64_t g_stride, int dtype, int64_t rows, int width, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0, "sigmoid_gate: bad sizes");
+  ALOFA_REQUIRE(!exact || dtype == kF32, "sigmoid_gate: the exact path is float32");
+  if (rows == 0) return 0;
+  const unsigned grid = blocks_of(rows * width);
+  if (exact) sigmoid_gate_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(x), x_stride, static_cast<const float*>(g), g_stride, rows, width);
+  else if (dtype == kF32) sigmoid_gate_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(x), x_stride, static_cast<const float*>(g), g_stride, rows, width);
+  else sigmoid_gate_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(x), x_stride, static_cast<const bf16_t*>(g), g_stride, rows, width);
+  return check_launch("sigmoid_gate");
+}
+
+extern "C" int alofa_add_channel_scaled(float* residual, const float* x, const float* scale, int64_t rows, int width, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && scale != nullptr, "add_channel_scaled: bad arguments");
+  if (rows == 0) return 0;
+  if (exact) add_channel_scaled_kernel<double><<<blocks_of(rows * width), 256, 0, stream>>>(residual, x, scale, rows * width, width);
+  else add_channel_scaled_kernel<float><<<blocks_of(rows * width), 256, 0, stream>>>(residual, x, scale, rows * width, width);
+  return check_launch("add_channel_scaled");
+}
+
+extern "C" int alofa_softcap(float* x, float cap, int64_t elements, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(elements >= 0 && cap > 0.f, "softcap: bad arguments");
+  if (elements == 0) return 0;
+  if (exact) softcap_kernel<double><<<blocks_of(elements), 256, 0, stream>>>(x, cap, elements);
+  else softcap_kernel<float><<<blocks_of(elements), 256, 0, stream>>>(x, cap, elements);
+  return check_launch("softcap");
+}
+
+extern "C" int alofa_relu_squared(void* out, int64_t out_stride, const void* x, int64_t x_stride, int dtype, int64_t rows, int width, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0, "relu_squared: bad sizes");
+  if (rows == 0) return 0;
+  if (dtype == kF32) relu_squared_kernel<float><<<blocks_of(rows * width), 256, 0, stream>>>(static_cast<float*>(out), out_stride, static_cast<const float*>(x), x_stride, rows, width);
+  else relu_squared_kernel<bf16_t><<<blocks_of(rows * width), 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(x), x_stride, rows, width);
+  return check_launch("relu_squared");
+}

@@ -88,6 +88,7 @@ class StepContext:
         self._slots: list = []
         self._memo: dict = {}
         self.token_store = fn.token_store
+        self.watch = fn.watch
         self.request_slots: Optional[torch.Tensor] = None   # int32 [entries] on the device: the request slot of every entry
         self.row_offsets: Optional[torch.Tensor] = None     # int32 [entries + 1] on the device: entry i owns the rows [i] .. [i+1]-1; None: one row each (decode graphs)
         self.want_slots: Optional[torch.Tensor] = None      # int32 [wanted rows] on the device: the request slot behind every wanted row
@@ -170,6 +171,7 @@ class StepFunction:
         self.steps_run = 0
         self.rows_run = 0
         self.last_context: Optional[StepContext] = None
+        self.watch = None                        # None, or a function (run entry, stream) called after every entry of a step that runs kernel by kernel
         # decode steps (one token per request) replay a captured HIP graph when every
         # part runs native kernels only; ALOFA_GRAPHS=0 switches that off
         self.use_graphs = os.environ.get("ALOFA_GRAPHS", "1") != "0" and model.capturable
@@ -429,7 +431,7 @@ class StepFunction:
         logit, and leaves the same in the token store at the row's request's slot.
         The buffer is re-used by the next step."""
         with ops.stream_scope():
-            if self.use_graphs and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            if self.use_graphs and self.watch is None and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
                 return self._run_decode_graph(entries, greedy)
             ctx, ids, rows = self.begin(entries)
             hidden = self.model.forward(ctx, ids)

@@ -25,6 +25,8 @@ def check_spec(spec: ModelSpec) -> None:
     for i, e in enumerate(spec.order):
         if not 0 <= e.layer < len(spec.layers):
             raise AlofaError("out_of_range", "run order names a layer that does not exist", f"entry={i} layer={e.layer}")
+        if e.join is not None and not 0 <= e.join < len(spec.joins):
+            raise AlofaError("out_of_range", "a run entry names a join that does not exist", f"entry={i} join={e.join} joins={len(spec.joins)}")
         if e.cache_of is not None:
             if not 0 <= e.cache_of < i or spec.order[e.cache_of].cache_of is not None:
                 raise AlofaError("invalid_argument", "an entry may read only the cache of an earlier entry that owns one", f"entry={i} cache_of={e.cache_of}")
@@ -33,6 +35,8 @@ def check_spec(spec: ModelSpec) -> None:
 def expected_tensors(spec: ModelSpec) -> dict:
     """name -> TensorRule for every tensor the model's parts read, in a fixed order."""
     out = dict(tensors_of("embedding", spec.embedding))
+    for join in spec.joins:
+        out.update(tensors_of("join", join))
     for layer in spec.layers:
         out.update(part_class("block", layer.block.kind).layer_tensors(layer))
     out.update(tensors_of("norm", spec.final_norm))
@@ -50,6 +54,7 @@ class Model:
         self.blocks = [part_class("block", l.block.kind)(l, weights, rt) for l in spec.layers]
         self.final_norm = build_part("norm", spec.final_norm, weights, rt)
         self.head = build_part("head", spec.head, weights, rt, embedding=self.embedding)
+        self.joins = [build_part("join", j, weights, rt) for j in spec.joins]
         self.order = list(spec.order)
 
     # What the cache manager has to provide. The blocks answer; an owner's key is (run entry, index
@@ -61,8 +66,12 @@ class Model:
 
     def state_needs(self) -> dict:
         """{(entry, k): StateNeed} for every mixer that carries state per request."""
-        return {(i, k): need for i, e in enumerate(self.order)
-                for k, need in enumerate(self.blocks[e.layer].state_needs()) if need is not None}
+        out = {(i, k): need for i, e in enumerate(self.order)
+               for k, need in enumerate(self.blocks[e.layer].state_needs()) if need is not None}
+        kept = getattr(self.embedding, "state_need", lambda: None)()      # (an embedding that looks one token back)
+        if kept is not None:
+            out[("embedding", 0)] = kept
+        return out
 
     def cache_owners(self) -> dict:
         """{(entry, k): the key whose cache that mixer uses} — its own, or the earlier entry's that
@@ -78,7 +87,8 @@ class Model:
 
     @property
     def capturable(self) -> bool:
-        return all(b.capturable for b in self.blocks)
+        return (all(b.capturable for b in self.blocks) and all(j.capturable for j in self.joins)
+                and getattr(self.embedding, "capturable", True))
 
     def prepare(self, n_positions: int) -> None:
         for b in self.blocks:
@@ -87,7 +97,7 @@ class Model:
     def weight_bytes(self) -> int:
         """Bytes of device memory the model's tensors take (a tensor shared by two parts counts once)."""
         seen, total = set(), 0
-        stack = [self.embedding, self.final_norm, self.head, *self.blocks]
+        stack = [self.embedding, self.final_norm, self.head, *self.joins, *self.blocks]
         while stack:
             part = stack.pop()
             for v in vars(part).values():
@@ -104,14 +114,24 @@ class Model:
         residual stream [T, hidden]."""
         hidden = self.embedding.forward(ctx, ids)
         rows, normed = hidden.shape[0], None
+        first = None
+        if self.joins:      # what the joins read beside the stream: the embedding's output, kept apart
+            first = ctx.scratch("hidden_first", tuple(hidden.shape), torch.float32)
+            first.copy_(hidden)
+        watch = getattr(ctx, "watch", None)      # (for tests and debugging: called with the stream after every run entry)
         for i, e in enumerate(self.order):
             block = self.blocks[e.layer]
-            if not block.takes_normed:
+            if e.join is not None:
+                self.joins[e.join].forward(ctx, hidden, first)
+                normed = None
+            if not block.takes_normed or watch is not None:
                 block.forward(ctx, i, hidden)
                 normed = None
+                if watch is not None:
+                    watch(i, hidden)
                 continue
             # the norm the next block starts with may be left by this block's last product (a launch less)
-            nxt = self.blocks[self.order[i + 1].layer] if i + 1 < len(self.order) else None
+            nxt = self.blocks[self.order[i + 1].layer] if i + 1 < len(self.order) and self.order[i + 1].join is None else None
             norm = nxt.wants_normed(rows) if nxt is not None and nxt.takes_normed else None
             then = (norm, ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)) if norm is not None and norm.as_rmsnorm() is not None else None
             normed = then[1] if block.forward(ctx, i, hidden, normed, then) else None

@@ -1,9 +1,11 @@
 """Architectures this engine knows. Importing the package registers them."""
 from ..config.registry import register_architecture
 from .qwen2 import Qwen2Config
+from .rerupel import RerupelConfig
 from .tugalix import TugalixConfig
 
 register_architecture(Qwen2Config.architecture, Qwen2Config)
 register_architecture(TugalixConfig.architecture, TugalixConfig)
+register_architecture(RerupelConfig.architecture, RerupelConfig)
 
-__all__ = ["Qwen2Config", "TugalixConfig"]
+__all__ = ["Qwen2Config", "RerupelConfig", "TugalixConfig"]

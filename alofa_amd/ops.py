@@ -1124,3 +1124,132 @@ def linear_recurrence(out: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: to
           _ptr(rows.slots), _ptr(rows.offsets), _I(rows.requests), _I(T), _I(heads), _I(dk), _I(dv), _I(decay_kind), _F(tau), _F(q_scale), _F(k_scale),
           _I(int(before_update)), _stream())
     return used.value
+
+
+# ------------------------------------------------------------- scaled sub-layers, pair embedding, stream joins, choices among experts
+
+def pair_embed(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0, store: Optional[torch.Tensor] = None,
+               pairs: Optional[torch.Tensor] = None, positions: Optional[torch.Tensor] = None, state: Optional[torch.Tensor] = None,
+               rows: Optional[RowsOfRequests] = None, buckets: int = 0, mul_prev: int = 0, mul_cur: int = 0) -> None:
+    """out[t] = table[ids[t]] * scale, plus, with ``pairs`` [buckets + 1, width], its row (before * mul_prev + id * mul_cur) mod
+    buckets, ``before`` being the request's token one place earlier: the row above in the step, or, for a request's first
+    row of the step, ``state[slot]`` (int32 [slots, 1]); a token at position 0 takes the row ``buckets``. The request's last
+    token of the step is left in ``state``. Ids below zero name tokens in ``store``, as for ``embed_gather``."""
+    _gpu("out", out, torch.float32, 2), _gpu("table", table, None, 2), _gpu("ids", ids, torch.int32, 1)
+    _contig("out", out), _contig("table", table), _contig("ids", ids)
+    T, h = out.shape
+    if table.shape[1] != h or ids.shape[0] != T:
+        raise AlofaError("shape_mismatch", "embedding width or token count does not fit", f"out={tuple(out.shape)} table={tuple(table.shape)} ids={tuple(ids.shape)}")
+    if store is not None:
+        _gpu("store", store, torch.int32, 1), _contig("store", store)
+    slots = offsets = req_of_row = None
+    if pairs is not None:
+        _gpu("pairs", pairs, table.dtype, 2), _contig("pairs", pairs), _gpu("positions", positions, torch.int32, 1), _contig("positions", positions)
+        _gpu("state", state, torch.int32), _contig("state", state)
+        if rows is None or tuple(pairs.shape) != (buckets + 1, h) or positions.shape[0] != T or rows.rows != T or buckets <= 0 or state.numel() < rows.n_slots:
+            raise AlofaError("shape_mismatch", "the pair table, positions, rows or state do not fit", f"pairs={tuple(pairs.shape)} buckets={buckets} tokens={T}")
+        slots, offsets, req_of_row = rows.slots, rows.offsets, rows.req_of_row
+    _call("alofa_pair_embed", _ptr(out), _ptr(table), _ptr(pairs), _I(dtype_code(table)), _ptr(ids), _ptr(positions), _ptr(state), _ptr(slots), _ptr(offsets),
+          _ptr(req_of_row), _I(T), _I(h), _ptr(store), _I(table.shape[0]), _F(scale), _L(buckets), _L(mul_prev), _L(mul_cur), _stream())
+
+
+def concat_rows(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
+    """out[t] = [a[t] | b[t]]: two float32 streams side by side in out's dtype."""
+    _gpu("out", out, None, 2), _gpu("a", a, torch.float32, 2), _gpu("b", b, torch.float32, 2), _contig("out", out), _contig("a", a), _contig("b", b)
+    if a.shape != b.shape or tuple(out.shape) != (a.shape[0], 2 * a.shape[1]):
+        raise AlofaError("shape_mismatch", "two streams of one shape, and an output twice as wide", f"out={tuple(out.shape)} a={tuple(a.shape)} b={tuple(b.shape)}")
+    _call("alofa_concat_rows", _ptr(out), _I(dtype_code(out)), _ptr(a), _ptr(b), _L(a.shape[0]), _I(a.shape[1]), _stream())
+
+
+def rmsnorm_spread(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, eps: float, pad: int, copies: int, exact: bool = False) -> None:
+    """out[t, k * pad + j] = rmsnorm(x[t])[j] * w[j] for k < copies (zeros for j from x's width up to pad). x float32 rows,
+    out rows of at least copies * pad values; row strides allowed."""
+    _gpu("out", out, None, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 1), _contig("w", w)
+    n, r = x.shape
+    if out.shape[0] != n or out.shape[1] != copies * pad or w.shape[0] != r or pad < r:
+        raise AlofaError("shape_mismatch", "the copies of the normed rows do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} pad={pad} copies={copies}")
+    _call("alofa_rmsnorm_spread", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(x), _L(_rows("x", x)), _ptr(w), _I(n), _I(r), _I(pad), _I(copies),
+          _F(eps), _I(int(exact)), _stream())
+
+
+def sigmoid_gate(x: torch.Tensor, g: torch.Tensor, exact: bool = False) -> None:
+    """x *= sigmoid(g), element by element on rows (row strides allowed)."""
+    _gpu("x", x, None, 2), _gpu("g", g, x.dtype, 2)
+    if x.shape != g.shape:
+        raise AlofaError("shape_mismatch", "gate and rows must agree", f"x={tuple(x.shape)} g={tuple(g.shape)}")
+    _call("alofa_sigmoid_gate", _ptr(x), _L(_rows("x", x)), _ptr(g), _L(_rows("g", g)), _I(dtype_code(x)), _L(x.shape[0]), _I(x.shape[1]), _I(int(exact)), _stream())
+
+
+def add_channel_scaled(residual: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, exact: bool = False) -> None:
+    """residual[t, c] += scale[c] * x[t, c], all float32."""
+    _gpu("residual", residual, torch.float32, 2), _gpu("x", x, torch.float32, 2), _gpu("scale", scale, torch.float32, 1)
+    _contig("residual", residual), _contig("x", x), _contig("scale", scale)
+    if x.shape != residual.shape or scale.shape[0] != residual.shape[1]:
+        raise AlofaError("shape_mismatch", "one factor per channel of the stream", f"residual={tuple(residual.shape)} x={tuple(x.shape)} scale={tuple(scale.shape)}")
+    _call("alofa_add_channel_scaled", _ptr(residual), _ptr(x), _ptr(scale), _L(residual.shape[0]), _I(residual.shape[1]), _I(int(exact)), _stream())
+
+
+def softcap_(x: torch.Tensor, cap: float, exact: bool = False) -> None:
+    """x = cap * tanh(x / cap) (float32, contiguous)."""
+    _gpu("x", x, torch.float32), _contig("x", x)
+    _call("alofa_softcap", _ptr(x), _F(cap), _L(x.numel()), _I(int(exact)), _stream())
+
+
+def relu_squared(out: torch.Tensor, x: torch.Tensor) -> None:
+    """out = max(x, 0)^2 on rows (row strides allowed; out may be x)."""
+    _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2)
+    if out.shape != x.shape:
+        raise AlofaError("shape_mismatch", "activation operands do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)}")
+    _call("alofa_relu_squared", _ptr(out), _L(_rows("out", out)), _ptr(x), _L(_rows("x", x)), _I(dtype_code(out)), _L(x.shape[0]), _I(x.shape[1]), _stream())
+
+
+MAX_EXPERTS = 512
+
+
+def route_top(z: torch.Tensor, dense: torch.Tensor, chosen: torch.Tensor, weights: torch.Tensor, top: int, scale: float = 1.0,
+              renormalize: bool = False, exact: bool = False) -> None:
+    """Per row of the router products z [T, E] (float32) the ``top`` largest (the lower index among equals):
+    ``chosen`` int32 [T, top] and ``weights`` float32 [T, top] = sigmoid(z) * scale (made to sum to one first with
+    ``renormalize``), in order of falling score; ``dense`` float32 [T, E] holds the same weights at the chosen places and 0 elsewhere."""
+    _gpu("z", z, torch.float32, 2), _gpu("dense", dense, torch.float32, 2), _gpu("chosen", chosen, torch.int32, 2), _gpu("weights", weights, torch.float32, 2)
+    for n, t in (("z", z), ("dense", dense), ("chosen", chosen), ("weights", weights)):
+        _contig(n, t)
+    T, E = z.shape
+    if tuple(dense.shape) != (T, E) or tuple(chosen.shape) != (T, top) or tuple(weights.shape) != (T, top) or not 0 < top <= E <= MAX_EXPERTS:
+        raise AlofaError("shape_mismatch", "the choice's outputs do not fit", f"z={tuple(z.shape)} dense={tuple(dense.shape)} chosen={tuple(chosen.shape)} top={top}")
+    _call("alofa_route_top", _ptr(z), _ptr(dense), _ptr(chosen), _ptr(weights), _I(T), _I(E), _I(top), _F(scale), _I(int(renormalize)), _I(int(exact)), _stream())
+
+
+def clamped_glu(act: torch.Tensor, g: torch.Tensor, u: torch.Tensor, dense: Optional[torch.Tensor], experts: int, ff: int, shared_ff: int,
+                limit: float, shared_limit: float, slope: float, exact: bool = False) -> None:
+    """act[t, c] = w a sigmoid(slope a) (b + 1), a = min(g, limit), b = clamp(u, -limit, limit), for the channels of ``experts``
+    experts of ``ff`` channels side by side (w = dense[t, expert]) and then ``shared_ff`` channels with w = 1 and a limit of their own."""
+    for n, t in (("act", act), ("g", g), ("u", u)):
+        _gpu(n, t, act.dtype, 2), _contig(n, t)
+    F = experts * ff + shared_ff
+    T = act.shape[0]
+    if tuple(g.shape) != (T, F) or tuple(u.shape) != (T, F) or act.shape[1] != F:
+        raise AlofaError("shape_mismatch", "gate, up and output are [rows, all experts' channels]", f"act={tuple(act.shape)} g={tuple(g.shape)} u={tuple(u.shape)} F={F}")
+    if experts:
+        _gpu("dense", dense, torch.float32, 2), _contig("dense", dense)
+        if tuple(dense.shape) != (T, experts):
+            raise AlofaError("shape_mismatch", "one weight per row and expert", f"dense={tuple(dense.shape)}")
+    _call("alofa_clamped_glu", _ptr(act), _ptr(g), _ptr(u), _I(dtype_code(act)), _ptr(dense if experts else None), _L(T), _I(experts), _I(ff), _I(shared_ff),
+          _F(limit), _F(shared_limit), _F(slope), _I(int(exact)), _stream())
+
+
+def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, scale: torch.Tensor, tmp: torch.Tensor, exact: bool = False) -> None:
+    """residual[t, c] += scale[c] * (a @ w.T)[t, c]; ``tmp`` float32 of the residual's shape takes the product on its way."""
+    gemm(tmp, a, w, exact=exact)
+    add_channel_scaled(residual, tmp, scale, exact)
+
+
+def head_project(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: bool = False) -> None:
+    """out[t, a, :] = w[a] @ x[t, a, :] for every head a: x [T, H * din] and out [T, H * dout] hold the heads side by side (row
+    strides allowed), w is [H, dout, din]."""
+    _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2), _gpu("w", w, None, 3), _contig("w", w)
+    H, dout, din = w.shape
+    if x.shape[0] != out.shape[0] or x.shape[1] != H * din or out.shape[1] != H * dout:
+        raise AlofaError("shape_mismatch", "the heads' rows do not fit their matrices", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)}")
+    for a in range(H):
+        gemm(out[:, a * dout:(a + 1) * dout], x[:, a * din:(a + 1) * din], w[a], exact=exact)

@@ -57,6 +57,51 @@ class RowPlan:
         return self._tiles[key]
 
 
+def paged_attend(ctx, entry, qkv, attn, heads, kv_heads, d, window, scale, position, rt) -> None:
+    """The rows of one step through attention over the pages of the mixer at ``entry``: ``qkv`` [T, (heads + 2 kv_heads) d] holds
+    the step's queries, keys and values, heads of one size d side by side; queries and keys take ``position``, keys and values go
+    to their rows' cache slots (where the mixer owns the cache), and ``attn`` [T, heads d] receives softmax(scale q k) v over the
+    keys each row may see. Which kernels run follows from the step's layout, the dtype and the sizes."""
+    T = qkv.shape[0]
+    exact = rt.exact
+    mfma_heads = d % 16 == 0
+    kv = ctx.kv(entry)
+    plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
+    table = position.table(ctx.n_positions)
+    if table is None:
+        hd = heads * d
+        position.apply(ctx, qkv[:, :hd].unflatten(1, (heads, d)),
+                            qkv[:, hd:hd + kv_heads * d].unflatten(1, (kv_heads, d)))
+        table = ctx.identity_rotation(d)
+    cos, sin = table
+    common = (heads, kv_heads, d, window, scale)
+    pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
+    fast_prefill = d in ops.PREFILL_HEAD_DIMS
+    # one new token per request: the decode kernel rotates it and writes its cache slot itself
+    fused = (not exact and pow2_pages and mfma_heads and kv.owner and ctx.max_q_len == 1 and plan.long_runs is None
+             and ops.can_fuse_rope_into_decode(d))
+    if fused:
+        pass
+    elif kv.owner:
+        ops.rope_kv_write(qkv, cos, sin, ctx.positions, heads, kv_heads, d, kv.slots, kv.k, kv.v)
+    else:
+        ops.rope_kv_write(qkv, cos, sin, ctx.positions, heads, kv_heads, d)
+    if exact or not pow2_pages or not mfma_heads or (plan.long_runs is not None and not fast_prefill):
+        # the exact path, and page or head sizes the bfloat16 kernels are not built for
+        ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
+    else:
+        if plan.long_runs is not None:      # portions of prompts
+            tiles, share, rows = plan.tiles(heads, kv_heads, d, window)
+            ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows)
+        if plan.n_short:                    # single tokens and very short portions, all query heads of a key head together
+            floats = ops.decode_scratch_floats(plan.n_short, heads, kv_heads, d, ctx.max_context, window)
+            partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
+            # (one token per request and nothing else in the step: token i is request i)
+            one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
+            ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
+                                 ctx.max_context, partial, rows=plan.short_rows, rope=(cos, sin, kv.slots) if fused else None)
+
+
 NAMES = {"q": "q_proj.weight", "k": "k_proj.weight", "v": "v_proj.weight", "o": "o_proj.weight",
          "q_bias": "q_proj.bias", "k_bias": "k_proj.bias", "v_bias": "v_proj.bias", "o_bias": "o_proj.bias"}
 
@@ -175,42 +220,8 @@ class GQAAttention(Mixer):
             ops.gemm(qkv, residual, self.w_qkv, self.b_qkv, norm=norm.as_rmsnorm())
         else:
             ops.gemm(qkv, x, self.w_qkv, self.b_qkv, exact=exact)
-        kv = ctx.kv(entry)
-        plan = ctx.memo("gqa_attention.rows", lambda: RowPlan(ctx))
-        table = self.position.table(ctx.n_positions)
-        if table is None:
-            hd = self.heads * self.d
-            self.position.apply(ctx, qkv[:, :hd].unflatten(1, (self.heads, self.d)),
-                                qkv[:, hd:hd + self.kv_heads * self.d].unflatten(1, (self.kv_heads, self.d)))
-            table = ctx.identity_rotation(self.d)
-        cos, sin = table
         attn = ctx.scratch("attn", (T, self.heads * self.d), self.rt.dtype)
-        common = (self.heads, self.kv_heads, self.d, self.window, self.scale)
-        pow2_pages = kv.k.shape[2] >= ops.MIN_FAST_PAGE and kv.k.shape[2] & (kv.k.shape[2] - 1) == 0
-        fast_prefill = self.d in ops.PREFILL_HEAD_DIMS
-        # one new token per request: the decode kernel rotates it and writes its cache slot itself
-        fused = (not exact and pow2_pages and self.mfma_heads and kv.owner and ctx.max_q_len == 1 and plan.long_runs is None
-                 and ops.can_fuse_rope_into_decode(self.d))
-        if fused:
-            pass
-        elif kv.owner:
-            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d, kv.slots, kv.k, kv.v)
-        else:
-            ops.rope_kv_write(qkv, cos, sin, ctx.positions, self.heads, self.kv_heads, self.d)
-        if exact or not pow2_pages or not self.mfma_heads or (plan.long_runs is not None and not fast_prefill):
-            # the exact path, and page or head sizes the bfloat16 kernels are not built for
-            ops.paged_attention(attn, qkv, kv.k, kv.v, kv.block_table, ctx.req_of_token, ctx.positions, *common, exact)
-        else:
-            if plan.long_runs is not None:      # portions of prompts
-                tiles, share, rows = plan.tiles(self.heads, self.kv_heads, self.d, self.window)
-                ops.attention_prefill(attn, qkv, kv.k, kv.v, kv.block_table, tiles, *common, share=share, rows=rows)
-            if plan.n_short:                    # single tokens and very short portions, all query heads of a key head together
-                floats = ops.decode_scratch_floats(plan.n_short, self.heads, self.kv_heads, self.d, ctx.max_context, self.window)
-                partial = ctx.scratch("attn_partial", (floats,), torch.float32) if floats else None
-                # (one token per request and nothing else in the step: token i is request i)
-                one_each = ctx.max_q_len == 1 and plan.short_rows is None and plan.long_runs is None
-                ops.attention_decode(attn, qkv, kv.k, kv.v, kv.block_table, None if one_each else ctx.req_of_token, ctx.positions, *common,
-                                     ctx.max_context, partial, rows=plan.short_rows, rope=(cos, sin, kv.slots) if fused else None)
+        paged_attend(ctx, entry, qkv, attn, self.heads, self.kv_heads, self.d, self.window, self.scale, self.position, self.rt)
         if out is not None:
             ops.gemm(out, attn, self.w_o, self.b_o, exact=exact)
         elif self.b_o is not None:

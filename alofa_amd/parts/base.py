@@ -15,7 +15,8 @@ dtype, ``residual`` the float32 residual stream):
   block         built from a LayerSpec; layer_tensors(layer); mixers() (the parts that may keep
                 a cache or state, in a fixed order); cache_needs(), state_needs(), capturable,
                 prepare(n_positions); forward(ctx, entry, hidden)  one layer on the stream
-  embedding     forward(ctx, ids) -> hidden[T,h] f32
+  embedding     forward(ctx, ids) -> hidden[T,h] f32; state_need() -> StateNeed | None (kept under the key ("embedding", 0))
+  join          forward(ctx, hidden[T,h] f32, first[T,h] f32)     the stream, replaced by a function of itself and the embedding's output
   head          forward(ctx, y[S,h]) -> logits[S,V] f32
 """
 from __future__ import annotations
@@ -28,7 +29,7 @@ import torch
 from ..config.base import PartSpec
 from ..errors import AlofaError
 
-FAMILIES = ("embedding", "norm", "position", "conv", "mixer", "feed_forward", "block", "head")
+FAMILIES = ("embedding", "norm", "position", "conv", "mixer", "feed_forward", "block", "head", "join")
 _REGISTRY = {f: {} for f in FAMILIES}
 
 
@@ -202,6 +203,16 @@ class FeedForward(Part):
     gives_normed = False      # as for a mixer: ``forward(..., then=(norm, rows))``
 
     def forward(self, ctx, x: torch.Tensor, residual: torch.Tensor) -> None:
+        raise NotImplementedError
+
+
+class Join(Part):
+    """What a run entry may ask for in front of it (``RunEntry.join``): the stream is replaced, where it lies, by a function
+    of itself and of the embedding's output, which the model keeps for it."""
+    family = "join"
+    capturable = False
+
+    def forward(self, ctx, hidden: torch.Tensor, first: torch.Tensor) -> None:
         raise NotImplementedError
 
 

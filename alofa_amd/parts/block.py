@@ -5,7 +5,10 @@ norms before their sub-layers, two residual sums in float32
 (src/alofa/model/arch/qwen.mojo:1418-1510). It reads the layer's parts
 ``mixer``, ``feed_forward`` and ``norms`` (two).
 
-filtered_prenorm: the same with a filter over time in front of every sub-layer, an optional feed-forward, and an
+scaled_prenorm: a += s0 * mixer(norm0(a)); a += s1 * feed_forward(norm1(a)), with s a vector per sub-layer (one factor per
+channel, times a factor for all) and an optional feed-forward.
+
+filtered_prenorm: the same as prenorm with a filter over time in front of every sub-layer, an optional feed-forward, and an
 optional weighted average over the outputs of all layers so far."""
 from __future__ import annotations
 
@@ -153,5 +156,63 @@ class FilteredPreNormBlock(Block):
             ops.depth_average(hidden, stack, self.depth_weights, self.level + 1, self.rt.exact)
 
 
+class ScaledPreNormBlock(Block):
+    """Pre-norm sub-layers whose results are multiplied channel by channel before they join the stream:
+    a += r * ls0 * mixer(norm0(a)), then, where the layer has a feed-forward, a += r * ls1 * feed_forward(norm1(a)).
+    It reads the layer's parts ``mixer``, ``norms`` (one per sub-layer) and ``feed_forward`` (may be None).
+    params: hidden, residual_scale (r), channel_scales (tensor names, one per sub-layer, each [hidden]; a name may be None).
+    A part that says ``takes_channel_scale`` is handed the vector (``scale=``) and applies it as it adds; any other part
+    leaves its result apart (``out=``) and the block adds it."""
+
+    @classmethod
+    def layer_tensors(cls, layer) -> dict:
+        out = {}
+        for n in layer.part("norms"):
+            out.update(tensors_of("norm", n))
+        out.update(tensors_of("mixer", layer.part("mixer")))
+        if layer.part("feed_forward") is not None:
+            out.update(tensors_of("feed_forward", layer.part("feed_forward")))
+        for name in layer.block.params["channel_scales"]:
+            if name is not None:
+                out[name] = TensorRule((layer.block.params["hidden"],), "norm")
+        return out
+
+    def __init__(self, layer, weights, rt):
+        super().__init__(layer, weights, rt)
+        p = layer.block.params
+        ff = layer.part("feed_forward")
+        subs = 1 if ff is None else 2
+        norms, names = layer.part("norms"), p["channel_scales"]
+        if len(norms) != subs or len(names) != subs:
+            raise AlofaError("invalid_argument", "one norm and one channel scale (or None) per sub-layer", f"prefix={layer.prefix} sub-layers={subs} norms={len(norms)} scales={len(names)}")
+        self.norms = [build_part("norm", n, weights, rt) for n in norms]
+        self.mixer = build_part("mixer", layer.part("mixer"), weights, rt)
+        self.feed_forward = build_part("feed_forward", ff, weights, rt) if ff is not None else None
+        r, h = float(p.get("residual_scale", 1.0)), int(p["hidden"])
+        # (the factor for all channels and the channels' own, multiplied once, in float64, and kept as float32)
+        self.scales = [rt.vector(((weights[n].double() if n is not None else torch.ones(h, dtype=torch.float64)) * r).float()) for n in names]
+        self.parts = [p for p in (*self.norms, self.mixer, self.feed_forward) if p is not None]
+
+    def mixers(self):
+        return self.mixer.stateful_parts()
+
+    def _add(self, ctx, part, hidden, scale, *args):
+        if getattr(part, "takes_channel_scale", False):
+            part.forward(ctx, *args, hidden, scale=scale)
+        else:
+            apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
+            part.forward(ctx, *args, hidden, out=apart)
+            ops.add_channel_scaled(hidden, apart, scale, self.rt.exact)
+
+    def forward(self, ctx, entry, hidden):
+        buf = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
+        self.norms[0].forward(buf, hidden)
+        self._add(ctx, self.mixer, hidden, self.scales[0], (entry, 0), buf)
+        if self.feed_forward is not None:
+            self.norms[1].forward(buf, hidden)
+            self._add(ctx, self.feed_forward, hidden, self.scales[1], buf)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "scaled_prenorm", ScaledPreNormBlock)
 register_part("block", "filtered_prenorm", FilteredPreNormBlock)

@@ -6,10 +6,13 @@ src/alofa/engine/executor.mojo:806-837). Gate and up run as one kernel that
 applies the activation before anything is written.
 
 Two matrices with an activation between them: down(act(up(x))), no biases. The activation xIELU has two numbers
-p, q of its own per layer: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2."""
+p, q of its own per layer: z > 0: softplus(p) z^2 + z/2; z <= 0: (1/2 + softplus(q)) (exp(z) - 1 - z) + z/2. The
+activation relu_squared is max(z, 0)^2 and has no tensor of its own."""
 from __future__ import annotations
 
 import math
+
+import torch
 
 from .. import ops
 from ..errors import AlofaError
@@ -63,32 +66,45 @@ def _softplus(z: float) -> float:
 
 
 class DenseActivated(FeedForward):
-    """params: prefix, hidden, intermediate, activation ("xielu"), names (after the prefix: up, down, act)."""
+    """params: prefix, hidden, intermediate, activation ("xielu" or "relu_squared"), names (after the prefix: up, down, and act for
+    xielu). ``forward(..., scale=)`` with a float32 vector: what is added to the stream is multiplied by it channel by channel."""
     capturable = True
+    takes_channel_scale = True
 
     @classmethod
     def tensors(cls, spec):
         p = spec.params
         pre, h, i, names = p["prefix"], p["hidden"], p["intermediate"], p["names"]
-        return {pre + names["up"]: TensorRule((i, h), "fan_in"), pre + names["down"]: TensorRule((h, i), "fan_in"), pre + names["act"]: TensorRule((2,), "bias")}
+        out = {pre + names["up"]: TensorRule((i, h), "fan_in"), pre + names["down"]: TensorRule((h, i), "fan_in")}
+        if p.get("activation", "xielu") == "xielu":
+            out[pre + names["act"]] = TensorRule((2,), "bias")
+        return out
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
         p = spec.params
-        if p.get("activation", "xielu") != "xielu":
+        self.activation = p.get("activation", "xielu")
+        if self.activation not in ("xielu", "relu_squared"):
             raise AlofaError("unsupported", "no such activation is built", f"activation={p['activation']}")
         self.hidden, self.intermediate = int(p["hidden"]), int(p["intermediate"])
         pre, names = p["prefix"], p["names"]
         self.w_up, self.w_down = rt.matrix(weights[pre + names["up"]]), rt.matrix(weights[pre + names["down"]])
-        # the two numbers are fixed once the weights are: what the kernel needs of them is formed here, in float64
-        pq = weights[pre + names["act"]].double().tolist()
-        self.a, self.b = _softplus(pq[0]), 0.5 + _softplus(pq[1])
+        if self.activation == "xielu":
+            # the two numbers are fixed once the weights are: what the kernel needs of them is formed here, in float64
+            pq = weights[pre + names["act"]].double().tolist()
+            self.a, self.b = _softplus(pq[0]), 0.5 + _softplus(pq[1])
 
-    def forward(self, ctx, x, residual):
+    def forward(self, ctx, x, residual, scale=None):
         act = ctx.scratch("ff_act", (residual.shape[0], self.intermediate), self.rt.dtype)
         ops.gemm(act, x, self.w_up, exact=self.rt.exact)
-        ops.activation(act, act, ops.XIELU, self.a, self.b, self.rt.exact)
-        ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
+        if self.activation == "xielu":
+            ops.activation(act, act, ops.XIELU, self.a, self.b, self.rt.exact)
+        else:
+            ops.relu_squared(act, act)
+        if scale is None:
+            ops.gemm(residual, act, self.w_down, add_to_out=True, exact=self.rt.exact)
+        else:
+            ops.gemm_channel_scaled(residual, act, self.w_down, scale, ctx.scratch("sub_out", tuple(residual.shape), torch.float32), self.rt.exact)
 
 
 register_part("feed_forward", "swiglu", SwiGLU)
