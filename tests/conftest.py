@@ -100,3 +100,16 @@ def tugalix_dirs(tmp_path_factory):
         write_random_model(cfg, d, seed=2000 + ord(name))
         out[name] = d
     return out
+
+
+@pytest.fixture(scope="session")
+def rerupel_dirs(tmp_path_factory):
+    """Model folders of the small Rerupel configurations, written by the engine's random-weights mode."""
+    from alofa_amd.weights import write_random_model
+    from rerupel_cases import RERUPEL
+    out = {}
+    for name, cfg in RERUPEL.items():
+        d = tmp_path_factory.mktemp(f"rerupel_{name}")
+        write_random_model(cfg, d, seed=3000 + ord(name))
+        out[name] = d
+    return out

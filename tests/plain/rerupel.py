@@ -165,8 +165,11 @@ def layer(x, w, cfg, i, store=_keep):
 def forward_hidden(w, cfg, ids, store=_keep) -> list:
     """The stream after every layer run, [T, h] each."""
     e = cfg["embedding"]
-    b = e["bigram"]
-    x0 = embed(ids, w["embed"], e["scale"], w["bigram"], b["buckets"], b["mul_prev"], b["mul_cur"])
+    b = e.get("bigram")
+    if b is None:      # (a model without the pair table)
+        x0 = w["embed"][np.asarray(ids)] * e["scale"]
+    else:
+        x0 = embed(ids, w["embed"], e["scale"], w["bigram"], b["buckets"], b["mul_prev"], b["mul_cur"])
     x, out = x0, []
     order, starts = run_order(cfg)
     for n, i in enumerate(order):
@@ -181,3 +184,39 @@ def forward_logits(w, cfg, ids, store=_keep) -> np.ndarray:
     x = forward_hidden(w, cfg, ids, store)[-1]
     z = store(rms_norm(x, w["final.norm"], cfg["norm"]["eps"])) @ w["embed"].T
     return soft_cap(z, cfg["logit_softcap"])
+
+
+def greedy(w, cfg, prompt, n_new) -> list:
+    """n_new tokens, each the first index of the highest logit after everything before it."""
+    ids, out = list(prompt), []
+    for _ in range(n_new):
+        out.append(int(np.argmax(forward_logits(w, cfg, ids)[-1])))
+        ids.append(out[-1])
+    return out
+
+
+def router_margins(w, cfg, ids) -> np.ndarray:
+    """Per position the smallest gap, over all runs of layers with a router, between the last router product that is taken
+    and the first that is not, in units of the products' spread at that position (infinite where nothing is left out).
+    Positions with a small gap are the ones where rounding may change which experts a token takes."""
+    T = len(ids)
+    out = np.full(T, np.inf)
+    e = cfg["embedding"]
+    b = e.get("bigram")
+    x0 = w["embed"][np.asarray(ids)] * e["scale"] if b is None else embed(ids, w["embed"], e["scale"], w["bigram"], b["buckets"], b["mul_prev"], b["mul_cur"])
+    x = x0
+    order, starts = run_order(cfg)
+    for n, i in enumerate(order):
+        if n in starts:
+            x = join_streams(x, x0, w["loop.in"])
+        l, p = cfg["layers"][i], f"l{i}."
+        if l["mlp"] is not None and l["mlp"]["kind"] == "moe" and l["mlp"]["router"]["top"] < l["mlp"]["router"]["experts"]:
+            mx = l["mixer"]
+            y = latent_attention(rms_norm(x, w[p + "norm1"], cfg["norm"]["eps"]), w[p + "mix.q"], w[p + "mix.dkv"], w[p + "mix.dkv.norm"], w[p + "mix.uk"],
+                                 w[p + "mix.uv"], w[p + "mix.g"], w[p + "mix.o"], mx["heads"], mx["dim"], mx["vdim"], mx["scale"], cfg["norm"]["eps"])
+            mid = x + cfg["residual_mult"] * (y * w[p + "ls1"])
+            z = np.sort(rms_norm(mid, w[p + "norm2"], cfg["norm"]["eps"]) @ w[p + "mlp.router"].T, axis=-1)[:, ::-1]
+            top = l["mlp"]["router"]["top"]
+            out = np.minimum(out, (z[:, top - 1] - z[:, top]) / (z.std(axis=-1) + 1e-30))
+        x = layer(x, w, cfg, i)
+    return out

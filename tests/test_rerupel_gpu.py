@@ -1,0 +1,248 @@
+"""Rerupel through the engine against the plain implementation, in float32 and bfloat16: whole prompts, the stream after
+every run of a layer, decoding token by token, portions down to two tokens, unequal requests in one batch, slots and pages
+that are used again, weights made so that one far key or the pair of tokens decides, and greedy generation through the
+engine's own loop."""
+import json
+
+import numpy as np
+import pytest
+
+from helpers import assert_close, bulk_and_tail, collect, mixed, portions, random_ids, whole
+from plain import rerupel as pr
+from rerupel_cases import RERUPEL, clear_calls, plain_logits, plain_model
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = ["float32", "bfloat16"]
+LENGTHS = {"A": 90, "B": 75, "C": 120, "D": 150, "E": 100}
+
+
+@pytest.fixture(scope="module")
+def replayers(rerupel_dirs):
+    from alofa_amd.replay import Replayer
+    made = {}
+
+    def get(name, dtype, max_tokens=512):
+        key = (name, dtype, max_tokens)
+        if key not in made:
+            made[key] = Replayer(rerupel_dirs[name], dtype, max_tokens, max_requests=4)
+        r = made[key]
+        assert not r.cache.requests, "a test left requests behind"
+        return r
+    return get
+
+
+def ids_of(name, seed=7, n=None):
+    return random_ids(seed, n or LENGTHS[name], RERUPEL[name]["vocab"])
+
+
+def compare(got, model_dir, ids, dtype, what):
+    rows = clear_calls(model_dir, ids, dtype)
+    assert len(rows) >= 0.6 * len(ids), f"{what}: too few positions are left to compare"
+    assert_close(np.asarray(got)[rows], plain_logits(model_dir, tuple(ids))[rows], dtype, what)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(RERUPEL))
+def test_whole_prompt(replayers, rerupel_dirs, name, dtype):
+    ids = ids_of(name)
+    got = collect(replayers(name, dtype), whole("w", ids))["w"]
+    compare(got, rerupel_dirs[name], ids, dtype, f"{name} whole")
+
+
+@pytest.mark.parametrize("name", ["A", "D", "E"])
+def test_the_stream_after_every_run_of_a_layer(replayers, rerupel_dirs, name):
+    """float32, run by run (a layer that is passed through several times counts every time)."""
+    ids = ids_of(name, n=33)
+    r = replayers(name, "float32")
+    seen = []
+    r.fn.watch = lambda i, hidden: seen.append(hidden.detach().cpu().numpy().astype(np.float64))
+    try:
+        collect(r, whole("w", ids))
+    finally:
+        r.fn.watch = None
+    cfg, w = plain_model(str(rerupel_dirs[name]))
+    want = pr.forward_hidden(w, cfg, ids)
+    assert len(seen) == len(want) == len(pr.run_order(cfg)[0])
+    for i, (a, b) in enumerate(zip(seen, want)):
+        assert np.abs(a - b).max() <= 1e-5 * max(1.0, np.abs(b).max()), f"run {i}"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(RERUPEL))
+def test_prompt_then_token_by_token(replayers, rerupel_dirs, name, dtype):
+    ids = ids_of(name)
+    got = collect(replayers(name, dtype), bulk_and_tail("t", ids, tail=40))["t"]
+    compare(got, rerupel_dirs[name], ids, dtype, f"{name} bulk+tail")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["B", "E"])
+def test_from_the_first_token_one_by_one(replayers, rerupel_dirs, name, dtype):
+    """Long decoding from nothing: single tokens only, the sequence's first token (which has no token before it) included."""
+    ids = ids_of(name, seed=3, n=70)
+    got = collect(replayers(name, dtype), bulk_and_tail("t", ids, tail=69))["t"]
+    compare(got, rerupel_dirs[name], ids, dtype, f"{name} one by one")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(RERUPEL))
+def test_portions_of_changing_size(replayers, rerupel_dirs, name, dtype):
+    ids = ids_of(name)
+    steps = portions("p", ids)
+    assert min(len(s["entries"][0]["tokens"]) for s in steps) == 2
+    got = collect(replayers(name, dtype), steps)["p"]
+    compare(got, rerupel_dirs[name], ids, dtype, f"{name} portions")
+    other = collect(replayers(name, dtype), portions("q", ids, sizes=(2, 19, 2, 2, 33, 3, 17)))["q"]
+    compare(other, rerupel_dirs[name], ids, dtype, f"{name} other portions")
+    if dtype == "float32":      # the cut changes nothing beyond rounding
+        assert np.abs(other - got).max() <= 2e-6 * max(1.0, np.abs(got).max())
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B", "D", "E"])
+def test_unequal_requests_together_with_slots_and_pages_used_again(rerupel_dirs, name, dtype):
+    """Up to four live requests, seven in all: portions beside single tokens, a request left out now and then; a slot and
+    its pages go to the next request as soon as one ends. Every request must come out as it does alone."""
+    from alofa_amd.replay import Replayer
+    vocab, top = RERUPEL[name]["vocab"], LENGTHS[name]
+    requests = {f"r{i}": random_ids(200 + i, n, vocab) for i, n in enumerate([top, 37, top - 23, 64, 35, top - 9, 50])}
+    steps, peak = mixed(requests, seed=9, tail=20)
+    assert max(len(s["entries"]) for s in steps) >= 3
+    r = Replayer(rerupel_dirs[name], dtype, peak, max_requests=4)
+    got = collect(r, steps)
+    r.cache.check()
+    assert not r.cache.requests
+    for req, ids in requests.items():
+        compare(got[req], rerupel_dirs[name], ids, dtype, f"{name} mixed {req}")
+
+
+def test_a_slot_used_again_starts_from_nothing(replayers, rerupel_dirs):
+    """The same request twice in the same slot, a different one between them: the token an earlier owner left in the slot,
+    and its pages, must not show."""
+    name = "A"
+    r = replayers(name, "float32")
+    a, b = ids_of(name, seed=1, n=40), ids_of(name, seed=2, n=55)
+    first = collect(r, whole("a", a))["a"]
+    collect(r, whole("b", b))
+    again = collect(r, portions("a", a, sizes=(3, 2, 9)))["a"]
+    assert np.abs(again - first).max() <= 2e-6 * max(1.0, np.abs(first).max())
+    assert_close(again, plain_logits(rerupel_dirs[name], tuple(a)), "float32", "slot used again")
+
+
+def _rewrite(model_dir, out_dir, change, config=None):
+    """A copy of a model folder with some tensors changed by ``change(name -> float32 tensor)``."""
+    import torch
+    from safetensors.torch import load_file, save_file
+    out_dir.mkdir(parents=True, exist_ok=True)
+    raw = json.loads((model_dir / "config.json").read_text())
+    if config is not None:
+        config(raw)
+    (out_dir / "config.json").write_text(json.dumps(raw))
+    w = {k: v.float() for k, v in load_file(str(model_dir / "model.safetensors")).items()}
+    change(w)
+    save_file({k: v.to(torch.bfloat16).contiguous() for k, v in w.items()}, str(out_dir / "model.safetensors"))
+    return out_dir
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_far_key_that_decides(rerupel_dirs, tmp_path, dtype):
+    """Queries and the keys' projections scaled up, so that single keys carry nearly all the weight, hundreds of tokens back
+    and across page borders, in a prompt's portions and in decoding."""
+    from alofa_amd.replay import Replayer
+    name = "A"
+
+    def sharpen(w):
+        for i in (0, 2):
+            w[f"l{i}.mix.q"] *= 5.0
+            w[f"l{i}.mix.uk"] *= 5.0
+    d = _rewrite(rerupel_dirs[name], tmp_path / "sharp", sharpen)
+    ids = ids_of(name, seed=21, n=330)
+    cfg, w = plain_model(str(d))
+    # (the weights do concentrate: the largest softmax weight of the last query, in the first layer's first head, is large)
+    b, m = cfg["embedding"]["bigram"], cfg["layers"][0]["mixer"]
+    hn = pr.rms_norm(pr.embed(ids, w["embed"], cfg["embedding"]["scale"], w["bigram"], b["buckets"], b["mul_prev"], b["mul_cur"]), w["l0.norm1"], cfg["norm"]["eps"])
+    c = pr.rms_norm(hn @ w["l0.mix.dkv"].T, w["l0.mix.dkv.norm"], cfg["norm"]["eps"])
+    s = (hn[-1] @ w["l0.mix.q"].T)[:m["dim"]] @ (c @ w["l0.mix.uk"].T)[:, :m["dim"]].T * m["scale"]
+    p = np.exp(s - s.max())
+    assert (p / p.sum()).max() > 0.5
+    r = Replayer(d, dtype, 384, max_requests=4)
+    got = collect(r, portions("p", ids, sizes=(150, 2, 61, 17, 3)))["p"]
+    compare(got, d, ids, dtype, "far key, portions")
+    got = collect(r, bulk_and_tail("t", ids, tail=40))["t"]
+    compare(got, d, ids, dtype, "far key, decoding")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_the_pair_of_tokens_decides(rerupel_dirs, tmp_path, dtype):
+    """The pair table scaled up until it outweighs the token's own row: a token before that is lost between two steps, or taken
+    from another request of the batch, shows in every logit."""
+    from alofa_amd.replay import Replayer
+    name = "E"
+
+    def loud(w):
+        w["bigram"] *= 8.0
+    d = _rewrite(rerupel_dirs[name], tmp_path / "pairs", loud)
+    ids = ids_of(name, seed=31, n=90)
+    r = Replayer(d, dtype, 512, max_requests=4)
+    got = collect(r, portions("p", ids, sizes=(2, 2, 5, 1, 1, 17, 3)))["p"]
+    compare(got, d, ids, dtype, "pairs, portions")
+    requests = {f"r{i}": random_ids(400 + i, n, RERUPEL[name]["vocab"]) for i, n in enumerate([60, 31, 47, 22, 38])}
+    steps, peak = mixed(requests, seed=3, tail=12)
+    got = collect(r, steps)
+    for req, seq in requests.items():
+        compare(got[req], d, seq, dtype, f"pairs, mixed {req}")
+
+
+def test_greedy_generation_through_the_engine(rerupel_dirs):
+    """The engine's own loop and scheduler: prompts of unequal length, more than a batch holds at once."""
+    from alofa_amd import Engine
+    for name in ("A", "C"):
+        cfg, w = plain_model(str(rerupel_dirs[name]))
+        prompts = [random_ids(300 + i, n, cfg["vocab"]) for i, n in enumerate((5, 23, 2, 41, 17, 9))]
+        want = [pr.greedy(w, cfg, p, 8) for p in prompts]
+        engine = Engine(rerupel_dirs[name], dtype="float32", max_tokens=64, max_batch=4, token_budget=48, max_chunk=16)
+        assert engine.generate(prompts, max_new=8) == want, name
+        engine.cache.check()
+        got = Engine(rerupel_dirs[name], dtype="bfloat16", max_tokens=64, max_batch=4).generate(prompts, max_new=8)
+        agree = sum(a == b for g, r in zip(got, want) for a, b in zip(g, r))
+        assert agree >= 36, f"{name}: {agree}/48 greedy tokens agree with the plain model in bfloat16"
+
+
+def test_decode_steps_replay_a_captured_graph(replayers, rerupel_dirs):
+    """Single-token steps run as a captured graph; every replay must move the token before on and fill the next slot of the pages."""
+    name = "A"
+    r = replayers(name, "bfloat16")
+    if not r.fn.use_graphs:
+        pytest.skip("graphs are switched off")
+    ids = ids_of(name, seed=5, n=60)
+    before = r.fn.graph_replays
+    got = collect(r, bulk_and_tail("t", ids, tail=30))["t"]
+    assert r.fn.graph_replays > before
+    compare(got, rerupel_dirs[name], ids, "bfloat16", "graph decode")
+
+
+def test_the_programs_take_the_design_by_its_config(rerupel_dirs, tmp_path):
+    """bin/generate and bin/trace_run on a folder of this design."""
+    import os
+    import subprocess
+    from conftest import ROOT
+    name = "A"
+    d = rerupel_dirs[name]
+    cfg, w = plain_model(str(d))
+    prompts = [random_ids(1, 5, cfg["vocab"]), random_ids(2, 19, cfg["vocab"])]
+    want = [pr.greedy(w, cfg, p, 5) for p in prompts]
+    env = dict(os.environ, ALOFA_WEIGHTS=str(d), ALOFA_DTYPE="float32", ALOFA_MAX_NEW="5", ALOFA_MAX_TOKENS="64",
+               ALOFA_PROMPT_IDS=";".join(",".join(map(str, p)) for p in prompts))
+    p = subprocess.run([str(ROOT / "bin" / "generate")], env=env, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert [[int(t) for t in line.split(",")] for line in p.stdout.strip().splitlines()] == want
+    ids = ids_of(name, seed=12, n=70)
+    steps = portions("a", ids, sizes=(33, 2, 1, 1, 20, 1))
+    text = "".join(json.dumps(s) + "\n" for s in steps)
+    p = subprocess.run([str(ROOT / "bin" / "trace_run"), "--model", str(d), "--dtype", "float32", "--out", str(tmp_path / "out"), "--max-tokens", "128"],
+                       input=text, capture_output=True, text=True, timeout=300)
+    assert p.returncode == 0, p.stderr[-2000:]
+    assert p.stdout.split("\n")[:-1] == [f"done {s['step']}" for s in steps]
+    got = np.concatenate([np.fromfile(tmp_path / "out" / f"{s['step']}.f32", dtype="<f4").reshape(-1, cfg["vocab"]) for s in steps])
+    assert_close(got, plain_logits(d, tuple(ids)), "float32", "program")
