@@ -1244,12 +1244,105 @@ def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor
     add_channel_scaled(residual, tmp, scale, exact)
 
 
-def head_project(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: bool = False) -> None:
+GR_STORE, GR_SIGMOID_GATE, GR_CLAMPED_GLU = 0, 1, 2
+
+
+def _grouped(out, out_step, x, x_step, w, w2, w_stride, w_step, n_out, K, last, rows, x_by_slot, tiles, tiles_per_batch, tile_batch, row_in,
+             gate, slot_weight, limit, limit_last, slope, epilogue) -> None:
+    last_batch, n_out_last, K_last = last if last is not None else (-1, n_out, K)
+    _call("alofa_grouped_product", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _L(out_step), _ptr(x), _L(_rows("x", x)), _L(x_step),
+          _ptr(w), _ptr(w2), _L(w_stride), _L(w_step), _I(n_out), _I(K), _I(last_batch), _I(n_out_last), _I(K_last), _I(rows), _I(int(x_by_slot)), _I(tiles),
+          _I(tiles_per_batch), _ptr(tile_batch), _ptr(row_in), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _ptr(slot_weight),
+          _F(limit), _F(limit_last), _F(slope), _I(epilogue), _stream())
+
+
+def _aligned_rows(t: torch.Tensor) -> bool:
+    return t.dtype is torch.bfloat16 and t.stride(-1) == 1 and t.stride(0) % 8 == 0 and t.data_ptr() % 16 == 0
+
+
+def head_project(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: bool = False, gate: Optional[torch.Tensor] = None) -> None:
     """out[t, a, :] = w[a] @ x[t, a, :] for every head a: x [T, H * din] and out [T, H * dout] hold the heads side by side (row
-    strides allowed), w is [H, dout, din]."""
+    strides allowed), w is [H, dout, din]. With ``gate`` (out's shape): out *= sigmoid(gate). bfloat16 rows whose heads start at
+    16-byte borders run as one launch on the matrix cores; everything else head by head through ``gemm``."""
     _gpu("out", out, None, 2), _gpu("x", x, out.dtype, 2), _gpu("w", w, None, 3), _contig("w", w)
     H, dout, din = w.shape
     if x.shape[0] != out.shape[0] or x.shape[1] != H * din or out.shape[1] != H * dout:
         raise AlofaError("shape_mismatch", "the heads' rows do not fit their matrices", f"out={tuple(out.shape)} x={tuple(x.shape)} w={tuple(w.shape)}")
+    if gate is not None:
+        _gpu("gate", gate, out.dtype, 2)
+        if gate.shape != out.shape:
+            raise AlofaError("shape_mismatch", "one gate per output", f"gate={tuple(gate.shape)} out={tuple(out.shape)}")
+    T = x.shape[0]
+    if not exact and out.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and din % 8 == 0 and _aligned_rows(x) and w.data_ptr() % 16 == 0 and T > 0:
+        per = (T + 15) // 16
+        _grouped(out, dout, x, din, w, None, din, dout * din, dout, din, None, T, False, H * per, per, None, None, gate, None, 0.0, 0.0, 0.0,
+                 GR_SIGMOID_GATE if gate is not None else GR_STORE)
+        return
     for a in range(H):
         gemm(out[:, a * dout:(a + 1) * dout], x[:, a * din:(a + 1) * din], w[a], exact=exact)
+    if gate is not None:
+        sigmoid_gate(out, gate, exact)
+
+
+class ExpertRows:
+    """The rows of a step sorted by the experts they take (``expert_rows``): ``row_in`` int32 [slots] (the row in a slot, -1: none),
+    ``slot_weight`` float32 [slots], ``slot_of`` int32 [T * top (+ T)] (the slot of row t's k-th choice; then, with a shared expert, of
+    row t's place in it), ``tile_batch`` int32 [tiles] (the expert of every 16 slots, -1: none)."""
+
+    def __init__(self, T: int, top: int, experts: int, shared: bool, scratch):
+        self.T, self.top, self.experts, self.shared = T, top, experts, shared
+        self.slots = (T * top + 15) // 16 * 16 + 16 * experts + ((T + 15) // 16 * 16 if shared else 0)
+        self.tiles = self.slots // 16
+        self.row_in, self.slot_weight = scratch("expert_row_in", (self.slots,), torch.int32), scratch("expert_slot_weight", (self.slots,), torch.float32)
+        self.slot_of, self.tile_batch = scratch("expert_slot_of", (T * (top + 1),), torch.int32), scratch("expert_tile_batch", (self.tiles,), torch.int32)
+
+
+def expert_rows(rows: ExpertRows, chosen: torch.Tensor, weights: torch.Tensor) -> None:
+    _gpu("chosen", chosen, torch.int32, 2), _gpu("weights", weights, torch.float32, 2), _contig("chosen", chosen), _contig("weights", weights)
+    if tuple(chosen.shape) != (rows.T, rows.top) or tuple(weights.shape) != (rows.T, rows.top):
+        raise AlofaError("shape_mismatch", "one choice and one weight per row and place", f"chosen={tuple(chosen.shape)} weights={tuple(weights.shape)}")
+    _call("alofa_expert_rows", _ptr(chosen), _ptr(weights), _ptr(rows.row_in), _ptr(rows.slot_weight), _ptr(rows.slot_of), _ptr(rows.tile_batch),
+          _I(rows.T), _I(rows.top), _I(rows.experts), _I(int(rows.shared)), _I(rows.slots), _I(rows.tiles), _stream())
+
+
+def can_group_experts(x: torch.Tensor, w_gate: torch.Tensor, ff: int, shared_ff: int) -> bool:
+    """Whether the experts' products can run slot by slot on the matrix cores: bfloat16, every reduction a multiple of eight."""
+    return (x.dtype is torch.bfloat16 and w_gate.dtype is torch.bfloat16 and _aligned_rows(x) and x.shape[1] % 8 == 0 and ff % 8 == 0 and shared_ff % 8 == 0)
+
+
+def experts_gate_up(act: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, rows: ExpertRows, ff: int, shared_ff: int,
+                    limit: float, shared_limit: float, slope: float) -> None:
+    """act[slot, :] = weight[slot] * a sigmoid(slope a) (b + 1) with a = min(gate_e(x[row]), limit), b = clamp(up_e(x[row]), -limit, limit)
+    for the expert e of the slot; w_gate and w_up hold the experts' matrices one below the other ([E * ff (+ shared_ff), h])."""
+    _gpu("act", act, torch.bfloat16, 2), _gpu("x", x, torch.bfloat16, 2), _gpu("w_gate", w_gate, torch.bfloat16, 2), _gpu("w_up", w_up, torch.bfloat16, 2)
+    _contig("w_gate", w_gate), _contig("w_up", w_up), _contig("act", act)
+    h = x.shape[1]
+    F = rows.experts * ff + (shared_ff if rows.shared else 0)
+    if tuple(w_gate.shape) != (F, h) or tuple(w_up.shape) != (F, h) or act.shape[0] < rows.slots or act.shape[1] < max(ff, shared_ff) or x.shape[0] != rows.T:
+        raise AlofaError("shape_mismatch", "the experts' matrices or the slots' rows do not fit", f"act={tuple(act.shape)} x={tuple(x.shape)} w_gate={tuple(w_gate.shape)} F={F}")
+    _grouped(act, 0, x, 0, w_gate, w_up, h, ff * h, ff, h, (rows.experts, shared_ff, h) if rows.shared else None, rows.slots, False, rows.tiles, 0,
+             rows.tile_batch, rows.row_in, None, rows.slot_weight, limit, shared_limit, slope, GR_CLAMPED_GLU)
+
+
+def experts_down(y: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, rows: ExpertRows, ff: int, shared_ff: int) -> None:
+    """y[slot, :] = down_e(act[slot, :]) (float32); w_down holds the experts' matrices side by side ([h, E * ff (+ shared_ff)])."""
+    _gpu("y", y, torch.float32, 2), _gpu("act", act, torch.bfloat16, 2), _gpu("w_down", w_down, torch.bfloat16, 2), _contig("w_down", w_down), _contig("y", y)
+    h = w_down.shape[0]
+    F = rows.experts * ff + (shared_ff if rows.shared else 0)
+    if w_down.shape[1] != F or tuple(y.shape) != (rows.slots, h) or act.shape[0] < rows.slots or not _aligned_rows(act) or F % 8:
+        raise AlofaError("shape_mismatch", "the experts' matrices or the slots' rows do not fit", f"y={tuple(y.shape)} act={tuple(act.shape)} w_down={tuple(w_down.shape)} F={F}")
+    _grouped(y, 0, act, 0, w_down, None, F, ff, h, ff, (rows.experts, h, shared_ff) if rows.shared else None, rows.slots, True, rows.tiles, 0,
+             rows.tile_batch, rows.row_in, None, None, 0.0, 0.0, 0.0, GR_STORE)
+
+
+def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale: Optional[torch.Tensor] = None) -> None:
+    """residual[t] += scale * (sum over row t's choices k, ascending, of y[slot of (t, k)], then its slot of the shared expert)."""
+    _gpu("residual", residual, torch.float32, 2), _gpu("y", y, torch.float32, 2), _contig("residual", residual), _contig("y", y)
+    T, h = residual.shape
+    if T != rows.T or tuple(y.shape) != (rows.slots, h):
+        raise AlofaError("shape_mismatch", "the slots' results do not fit the stream", f"residual={tuple(residual.shape)} y={tuple(y.shape)}")
+    if scale is not None:
+        _gpu("scale", scale, torch.float32, 1), _contig("scale", scale)
+        if scale.shape[0] != h:
+            raise AlofaError("shape_mismatch", "one factor per channel of the stream", f"scale={tuple(scale.shape)}")
+    _call("alofa_experts_sum", _ptr(residual), _ptr(y), _ptr(rows.slot_of), _ptr(scale), _I(T), _I(h), _I(rows.top), _I(int(rows.shared)), _stream())

@@ -98,9 +98,7 @@ class LatentAttention(Mixer):
         attn = ctx.scratch("attn", (T, H * d), self.rt.dtype)
         paged_attend(ctx, where, qkv, attn, H, 1, d, self.window, self.scale, self.position, self.rt)
         heads_out = ctx.scratch("latent_out", (T, H * self.dv), self.rt.dtype)
-        ops.head_project(heads_out, attn, self.w_result, exact)
-        if self.gated:
-            ops.sigmoid_gate(heads_out, qg[:, H * self.dk:], exact)
+        ops.head_project(heads_out, attn, self.w_result, exact, gate=qg[:, H * self.dk:] if self.gated else None)
         if out is not None:
             ops.gemm(out, heads_out, self.w_o, exact=exact)
         elif scale is None:

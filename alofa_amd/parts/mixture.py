@@ -9,12 +9,17 @@ The experts' matrices lie side by side in one tensor each (gate and up by rows, 
 last), so that every expert is a slice of them."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .. import ops
 from ..errors import AlofaError
 from ..weights.loader import TensorRule
 from .base import FeedForward, register_part
+
+
+SPARSE_EXPERTS = os.environ.get("ALOFA_SPARSE_EXPERTS", "1") != "0"      # 0 (for measurements): every expert against every row
 
 
 class RoutedExperts(FeedForward):
@@ -75,9 +80,24 @@ class RoutedExperts(FeedForward):
         ops.route_top(z, dense, chosen, weights, self.top, self.weight_scale, self.renormalize, self.rt.exact)
         return dense, chosen, weights
 
+    def sparse(self, x) -> bool:
+        """Whether the experts run slot by slot (every row against the experts it takes only) rather than all of them against
+        every row with weights of zero: where a token leaves at least half of the experts out, and the kernel takes the sizes."""
+        return (SPARSE_EXPERTS and not self.rt.exact and 2 * self.top <= self.experts
+                and ops.can_group_experts(x, self.w_gate, self.ff, self.shared_ff))
+
     def forward(self, ctx, x, residual, scale=None):
         T, exact = residual.shape[0], self.rt.exact
         dense, chosen, weights = self.route(ctx, x)
+        if self.sparse(x):
+            rows = ops.ExpertRows(T, self.top, self.experts, self.shared_ff > 0, ctx.scratch)
+            ops.expert_rows(rows, chosen, weights)
+            act = ctx.scratch("experts_act", (rows.slots, (max(self.ff, self.shared_ff) + 7) // 8 * 8), torch.bfloat16)
+            ops.experts_gate_up(act, x, self.w_gate, self.w_up, rows, self.ff, self.shared_ff, self.limit, self.shared_limit, self.slope)
+            y = ctx.scratch("experts_out", (rows.slots, self.hidden), torch.float32)
+            ops.experts_down(y, act, self.w_down, rows, self.ff, self.shared_ff)
+            ops.experts_sum(residual, y, rows, scale)
+            return
         # every expert's gate and up for every row, the rows an expert is not taken by weighted with zero
         g, u = ctx.scratch("experts_gate", (T, self.channels), self.rt.dtype), ctx.scratch("experts_up", (T, self.channels), self.rt.dtype)
         ops.gemm(g, x, self.w_gate, exact=exact)

@@ -190,3 +190,53 @@ def test_a_projection_per_head(heads, din, dout, rows, dtype):
     got = out.float().cpu().numpy()
     assert np.abs(got[:, 8:] - want).max() <= (1e-5 if exact else 2e-2) * max(1.0, np.abs(want).max())
     assert (got[:, :8] == 5.0).all()
+
+
+@pytest.mark.parametrize("T, h, E, top, ff, sff", [(21, 40, 5, 2, 16, 24), (1, 64, 8, 3, 96, 96), (150, 72, 16, 4, 8, 0), (64, 48, 4, 1, 40, 8), (5, 200, 3, 1, 24, 48)])
+def test_routed_experts_slot_by_slot(T, h, E, top, ff, sff):
+    """The rows sorted by expert and every expert against its own rows only, against the plain sum over the experts a token
+    takes; every row lands in exactly one slot per choice."""
+    from alofa_amd import ops
+    rng = np.random.default_rng(T)
+    bf = torch.bfloat16
+    hn = b16(rng.normal(0, 1, (T, h)))
+    experts = [tuple(b16(rng.normal(0, s, shape)) for s, shape in ((0.3, (ff, h)), (0.3, (ff, h)), (0.3, (h, ff)))) for _ in range(E)]
+    shared = tuple(b16(rng.normal(0, s, shape)) for s, shape in ((0.3, (sff, h)), (0.3, (sff, h)), (0.3, (h, sff)))) if sff else None
+    w_router = b16(rng.normal(0, 0.5, (E, h)))
+    want = pr.routed_experts(hn, w_router, experts, shared, top, 1.5, 1.0, 0.6)
+    x = dev(hn, bf)
+    z = torch.empty(T, E, device=DEV)
+    ops.gemm(z, x, dev(w_router, bf))
+    dense, chosen, weights = torch.empty(T, E, device=DEV), torch.empty(T, top, dtype=torch.int32, device=DEV), torch.empty(T, top, device=DEV)
+    ops.route_top(z, dense, chosen, weights, top, 1.5, False, False)
+    both = experts + ([shared] if sff else [])
+    w_gate, w_up = (dev(np.concatenate([e[k] for e in both], axis=0), bf) for k in (0, 1))
+    w_down = dev(np.concatenate([e[2] for e in both], axis=1), bf)
+    assert ops.can_group_experts(x, w_gate, ff, sff)
+    rows = ops.ExpertRows(T, top, E, sff > 0, lambda name, shape, dtype: torch.empty(shape, dtype=dtype, device=DEV))
+    ops.expert_rows(rows, chosen, weights)
+    row_in, slot_of, tile_batch = rows.row_in.cpu().numpy(), rows.slot_of.cpu().numpy(), rows.tile_batch.cpu().numpy()
+    picks = chosen.cpu().numpy()
+    for t in range(T):
+        for k in range(top):
+            slot = slot_of[t * top + k]
+            assert row_in[slot] == t and tile_batch[slot // 16] == picks[t, k]
+        if sff:
+            assert row_in[slot_of[T * top + t]] == t and tile_batch[slot_of[T * top + t] // 16] == E
+    assert (row_in >= 0).sum() == T * (top + (1 if sff else 0))
+    act = torch.zeros(rows.slots, (max(ff, sff) + 7) // 8 * 8, dtype=bf, device=DEV)
+    ops.experts_gate_up(act, x, w_gate, w_up, rows, ff, sff, 1.0, 0.6, 1.702)
+    y = torch.empty(rows.slots, h, device=DEV)
+    ops.experts_down(y, act, w_down, rows, ff, sff)
+    stream = rng.normal(0, 1, (T, h)).astype(np.float32)
+    scale = rng.normal(1, 0.3, h).astype(np.float32)
+    out = dev(stream)
+    ops.experts_sum(out, y, rows, dev(scale))
+    got = (out.cpu().numpy().astype(np.float64) - stream) / scale
+    assert np.abs(got - want).max() <= 3e-2 * max(1.0, np.abs(want).max())
+    again = dev(stream)      # the same rows in another order of arrival give the same bits
+    ops.expert_rows(rows, chosen, weights)
+    ops.experts_gate_up(act, x, w_gate, w_up, rows, ff, sff, 1.0, 0.6, 1.702)
+    ops.experts_down(y, act, w_down, rows, ff, sff)
+    ops.experts_sum(again, y, rows, dev(scale))
+    assert torch.equal(again, out)
