@@ -9,7 +9,10 @@ Uv_a (sum_j p_j c_j), every head asks the same keys and values, the latents them
 channels, and its result is taken through Uv_a afterwards: attention with H query heads over ONE key/value head of size r,
 which is what the paged attention kernels of this package do best (all heads of a key head share the keys a block reads).
 The cache holds c twice, as keys [page, 1, slot, d] and as transposed values [page, 1, d, slot] (d: r widened to a size
-the kernels are built for, with zeros), the layouts those kernels read."""
+the kernels are built for, with zeros), the layouts those kernels read.
+
+A latent wider than the largest head the kernels take cannot be a head: there the keys and values of every head are formed
+from c when it is made (k_a = Uk_a c, v_a = Uv_a c) and kept per head in the pages, as for any attention with H key heads."""
 from __future__ import annotations
 
 import torch
@@ -27,7 +30,8 @@ NAMES = {"q": "q", "down": "down", "up_k": "up_k", "up_v": "up_v", "gate": "gate
 class LatentAttention(Mixer):
     """params: prefix, hidden, heads, head_dim, v_head_dim, latent (r), scale (None: 1/sqrt(head_dim)), latent_norm (PartSpec of
     the norm of the latent, an RMSNorm), gate ("sigmoid" or None), window (None or a count of keys), names (tensor names after the
-    prefix for q, down, up_k, up_v, gate, o). ``forward(..., scale=)`` with a float32 vector: what is added to the stream is
+    prefix for q, down, up_k, up_v, gate, o); optional: keep ("latent", the default: the pages hold the latent where the kernels take
+    its size; "heads": they hold every head's keys and values). ``forward(..., scale=)`` with a float32 vector: what is added to the stream is
     multiplied by it channel by channel."""
     capturable = True
     takes_channel_scale = True
@@ -52,53 +56,94 @@ class LatentAttention(Mixer):
         self.window = p.get("window")
         if p.get("gate") not in (None, "sigmoid"):
             raise AlofaError("unsupported", "no such gate is built", f"gate={p['gate']}")
-        # the one head size of the attention kernels: the latent's, widened to a size they are built for
-        self.d = GQAAttention.common_head_size(self.r, self.r)
-        if self.d not in ops.PREFILL_HEAD_DIMS:
-            self.d = next((s for s in ops.PREFILL_HEAD_DIMS if s >= self.d), self.d)
-        if self.d > ops.MAX_HEAD_DIM:
-            raise AlofaError("unsupported", f"the attention kernels take latents of up to {ops.MAX_HEAD_DIM} channels", f"latent={self.r}")
-        H, dk, dv, r, d = self.heads, self.dk, self.dv, self.r, self.d
+        H, dk, dv, r = self.heads, self.dk, self.dv, self.r
         self.scale = float(p["scale"]) if p.get("scale") is not None else dk ** -0.5
-        mats = [weights[pre + n["q"]]] + ([weights[pre + n["gate"]]] if p.get("gate") is not None else [])
-        if len({m.dtype for m in mats}) > 1:
-            mats = [m.float() for m in mats]
         self.gated = p.get("gate") is not None
-        self.w_in = rt.matrix(torch.cat(mats, dim=0))          # queries and gates in one product
-        self.w_down = rt.matrix(weights[pre + n["down"]])
         norm = p.get("latent_norm")
         self.norm = build_part("norm", norm, weights, rt).as_rmsnorm() if norm is not None else None
         if self.norm is None:
             raise AlofaError("unsupported", "the latent's norm is an RMSNorm", f"norm={norm.kind if norm is not None else None}")
-        # per head [out, in]: a query into the latent's channels (Uk_a^T, [d, dk], zero rows beyond r) and a result out of them (Uv_a, [dv, d], zero columns beyond r)
-        uk = weights[pre + n["up_k"]].reshape(H, dk, r).transpose(1, 2)
-        self.w_query = rt.matrix(torch.cat([uk, torch.zeros(H, d - r, dk, dtype=uk.dtype)], dim=1).contiguous())
-        uv = weights[pre + n["up_v"]].reshape(H, dv, r)
-        self.w_result = rt.matrix(torch.cat([uv, torch.zeros(H, dv, d - r, dtype=uv.dtype)], dim=2).contiguous())
-        self.w_o = rt.matrix(weights[pre + n["o"]])
+        self.w_down = rt.matrix(weights[pre + n["down"]])
+        # the one head size of the attention kernels: the latent's, widened to a size they are built for
+        d = GQAAttention.common_head_size(r, r)
+        if d not in ops.PREFILL_HEAD_DIMS:
+            d = next((s for s in ops.PREFILL_HEAD_DIMS if s >= d), d)
+        self.latent_heads = d <= ops.MAX_HEAD_DIM and p.get("keep", "latent") == "latent"
+        w_q, w_g, w_o = weights[pre + n["q"]], weights[pre + n["gate"]] if self.gated else None, weights[pre + n["o"]]
+        if self.latent_heads:
+            # per head [out, in]: a query into the latent's channels (Uk_a^T, [d, dk], zero rows beyond r) and a result out of them (Uv_a, [dv, d], zero columns beyond r)
+            uk = weights[pre + n["up_k"]].reshape(H, dk, r).transpose(1, 2)
+            self.w_query = rt.matrix(torch.cat([uk, torch.zeros(H, d - r, dk, dtype=uk.dtype)], dim=1).contiguous())
+            uv = weights[pre + n["up_v"]].reshape(H, dv, r)
+            self.w_result = rt.matrix(torch.cat([uv, torch.zeros(H, dv, d - r, dtype=uv.dtype)], dim=2).contiguous())
+            self.kv_heads = 1
+        else:
+            # keys and values per head, every head widened to one size with zero rows (zero columns of the output matrix)
+            d = GQAAttention.common_head_size(dk, dv)
+            if d > ops.MAX_HEAD_DIM:
+                raise AlofaError("unsupported", f"the attention kernels take heads of up to {ops.MAX_HEAD_DIM} channels", f"head_dim={dk} v_head_dim={dv}")
+            w_q = _padded_heads(w_q, H, dk, d)
+            self.w_kv = rt.matrix(torch.cat([_padded_heads(weights[pre + n["up_k"]], H, dk, d), _padded_heads(weights[pre + n["up_v"]], H, dv, d)], dim=0))
+            if d != dv:
+                w_g = _padded_heads(w_g, H, dv, d) if self.gated else None
+                w_o = _padded_heads(w_o.t(), H, dv, d).t()
+            self.kv_heads = H
+        self.d = d
+        self.w_q = rt.matrix(w_q)
+        self.w_gate = rt.matrix(w_g) if self.gated else None
+        if self.gated and self.latent_heads and w_q.dtype is w_g.dtype:      # queries and gates in one product
+            self.w_in = rt.matrix(torch.cat([w_q, w_g], dim=0))
+        else:
+            self.w_in = None
+        self.w_o = rt.matrix(w_o)
         self.position = build_part("position", PartSpec("none", {"head_dim": d}), weights, rt)
 
     def cache_need(self):
-        return CacheNeed.keys_and_values(1, self.d, self.window)
+        return CacheNeed.keys_and_values(self.kv_heads, self.d, self.window)
 
     def prepare(self, n_positions):
         self.position.table(n_positions)
 
+    def _latent(self, ctx, x, out, pad, copies):
+        """The step's latents, normed, ``copies`` times side by side in ``out`` (each widened to ``pad`` channels with zeros)."""
+        down = ctx.scratch("latent_down", (x.shape[0], self.r), torch.float32)
+        ops.gemm(down, x, self.w_down, exact=self.rt.exact)
+        w, eps = self.norm
+        ops.rmsnorm_spread(out, down, w, eps, pad, copies, self.rt.exact)
+
     def forward(self, ctx, where, x, residual, scale=None, out=None):
         T, exact, H, d = residual.shape[0], self.rt.exact, self.heads, self.d
-        qg = ctx.scratch("latent_in", (T, self.w_in.shape[0]), self.rt.dtype)
-        ops.gemm(qg, x, self.w_in, exact=exact)
-        down = ctx.scratch("latent_down", (T, self.r), torch.float32)
-        ops.gemm(down, x, self.w_down, exact=exact)
-        # [a query per head | the latent as key | the latent as value]
-        qkv = ctx.scratch("qkv", (T, (H + 2) * d), self.rt.dtype)
-        w, eps = self.norm
-        ops.rmsnorm_spread(qkv[:, H * d:], down, w, eps, d, 2, exact)
-        ops.head_project(qkv[:, :H * d], qg[:, :H * self.dk], self.w_query, exact)
         attn = ctx.scratch("attn", (T, H * d), self.rt.dtype)
-        paged_attend(ctx, where, qkv, attn, H, 1, d, self.window, self.scale, self.position, self.rt)
-        heads_out = ctx.scratch("latent_out", (T, H * self.dv), self.rt.dtype)
-        ops.head_project(heads_out, attn, self.w_result, exact, gate=qg[:, H * self.dk:] if self.gated else None)
+        if self.latent_heads:
+            if self.w_in is not None:
+                qg = ctx.scratch("latent_in", (T, self.w_in.shape[0]), self.rt.dtype)
+                ops.gemm(qg, x, self.w_in, exact=exact)
+                q, gate = qg[:, :H * self.dk], qg[:, H * self.dk:]
+            else:
+                q, gate = ctx.scratch("latent_q", (T, H * self.dk), self.rt.dtype), None
+                ops.gemm(q, x, self.w_q, exact=exact)
+                if self.gated:
+                    gate = ctx.scratch("latent_gate", (T, H * self.dv), self.rt.dtype)
+                    ops.gemm(gate, x, self.w_gate, exact=exact)
+            # [a query per head | the latent as key | the latent as value]
+            qkv = ctx.scratch("qkv", (T, (H + 2) * d), self.rt.dtype)
+            self._latent(ctx, x, qkv[:, H * d:], d, 2)
+            ops.head_project(qkv[:, :H * d], q, self.w_query, exact)
+            paged_attend(ctx, where, qkv, attn, H, 1, d, self.window, self.scale, self.position, self.rt)
+            heads_out = ctx.scratch("latent_out", (T, H * self.dv), self.rt.dtype)
+            ops.head_project(heads_out, attn, self.w_result, exact, gate=gate)
+        else:
+            qkv = ctx.scratch("qkv", (T, 3 * H * d), self.rt.dtype)
+            ops.gemm(qkv[:, :H * d], x, self.w_q, exact=exact)
+            c = ctx.scratch("latent", (T, self.r), self.rt.dtype)
+            self._latent(ctx, x, c, self.r, 1)
+            ops.gemm(qkv[:, H * d:], c, self.w_kv, exact=exact)
+            paged_attend(ctx, where, qkv, attn, H, H, d, self.window, self.scale, self.position, self.rt)
+            if self.gated:
+                gate = ctx.scratch("latent_gate", (T, H * d), self.rt.dtype)
+                ops.gemm(gate, x, self.w_gate, exact=exact)
+                ops.sigmoid_gate(attn, gate, exact)
+            heads_out = attn
         if out is not None:
             ops.gemm(out, heads_out, self.w_o, exact=exact)
         elif scale is None:

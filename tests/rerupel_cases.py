@@ -56,6 +56,11 @@ RERUPEL = {
         (_latent(5, 15, 9, 10, 0.3), _dense(30)),
         (_latent(1, 30, 50, 18, 0.2), _moe(5, 2, 0.8, 14, 1.25, (6, 4.0))),
         (_latent(10, 6, 10, 34, 0.4), _moe(2, 1, 3.0, 22, 0.9))]),
+    # latents wider than any head the attention kernels take (the pages then hold every head's keys and values), values wider
+    # and narrower than keys
+    "F": _config(150, 64, 1e-6, 0.6, 25.0, 4.0, (89, 3, 11), (0, 2, 2), [
+        (_latent(2, 16, 24, 264, 0.25), _dense(48)),
+        (_latent(3, 32, 16, 320, 0.18), _moe(4, 2, 1.0, 16, 2.0, (16, 2.0)))]),
 }
 
 

@@ -14,7 +14,7 @@ from rerupel_cases import RERUPEL, clear_calls, plain_logits, plain_model
 pytestmark = pytest.mark.gpu
 
 DTYPES = ["float32", "bfloat16"]
-LENGTHS = {"A": 90, "B": 75, "C": 120, "D": 150, "E": 100}
+LENGTHS = {"A": 90, "B": 75, "C": 120, "D": 150, "E": 100, "F": 80}
 
 
 @pytest.fixture(scope="module")
@@ -100,7 +100,7 @@ def test_portions_of_changing_size(replayers, rerupel_dirs, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "D", "E", "F"])
 def test_unequal_requests_together_with_slots_and_pages_used_again(rerupel_dirs, name, dtype):
     """Up to four live requests, seven in all: portions beside single tokens, a request left out now and then; a slot and
     its pages go to the next request as soon as one ends. Every request must come out as it does alone."""
