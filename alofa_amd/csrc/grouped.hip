@@ -39,11 +39,12 @@ __device__ __forceinline__ bf16x8 grouped_frag(const bf16_t* __restrict__ p, boo
   return __builtin_bit_cast(bf16x8, v);
 }
 
-template <int NC, int kEpilogue, typename TO>
+template <int RT, int NC, int kEpilogue, typename TO>
 __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                                                               const bf16_t* __restrict__ W2, const int32_t* __restrict__ tile_batch,
                                                               const int32_t* __restrict__ row_in, const bf16_t* __restrict__ gate,
                                                               const float* __restrict__ slot_weight, GroupedShape s, int col_groups) {
+  // RT: 16-row tiles a wavefront takes together (a tile is then 16 * RT rows): a fragment of the matrix serves them all
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
   const int64_t task = static_cast<int64_t>(blockIdx.x) * 4 + wave;
   const int tile = static_cast<int>(task / col_groups), cg = static_cast<int>(task % col_groups);
@@ -51,10 +52,10 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
   int batch, slot0;
   if (s.tiles_per_batch > 0) {
     batch = tile / s.tiles_per_batch;
-    slot0 = (tile % s.tiles_per_batch) * 16;
+    slot0 = (tile % s.tiles_per_batch) * 16 * RT;
   } else {
     batch = tile_batch[tile];
-    slot0 = tile * 16;
+    slot0 = tile * 16 * RT;
   }
   if (batch < 0) return;
   const bool last = batch == s.last_batch;
@@ -62,66 +63,87 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
   const int o0 = cg * NC * 16;
   if (o0 >= n_out) return;
   const int r = lane % 16, kq = (lane / 16) * 8;
-  const int slot = slot0 + r;
-  int row = -1;
-  if (slot < s.rows) row = row_in ? row_in[slot] : slot;
-  const bf16_t* xr = x + static_cast<int64_t>(row < 0 ? 0 : (s.x_by_slot ? slot : row)) * s.x_stride + batch * s.x_batch_step;
-  const bf16_t* wb = W + batch * s.w_batch_step, *wb2 = kEpilogue == kGrClampedGlu ? W2 + batch * s.w_batch_step : nullptr;
-  f32x4 acc[NC], acc2[NC];
+  int row[RT];
+  const bf16_t* xr[RT];
+  bool any = false;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) acc[c] = acc2[c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = 0; t < RT; ++t) {
+    const int slot = slot0 + t * 16 + r;
+    row[t] = -1;
+    if (slot < s.rows) row[t] = row_in ? row_in[slot] : slot;
+    xr[t] = x + static_cast<int64_t>(row[t] < 0 ? 0 : (s.x_by_slot ? slot : row[t])) * s.x_stride + batch * s.x_batch_step;
+    any = any || row[t] >= 0;
+  }
+  if (!__any(any)) return;
+  const bf16_t* wb = W + batch * s.w_batch_step, *wb2 = kEpilogue == kGrClampedGlu ? W2 + batch * s.w_batch_step : nullptr;
+  f32x4 acc[RT][NC], acc2[RT][NC];
+#pragma unroll
+  for (int t = 0; t < RT; ++t)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) acc[t][c] = acc2[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
   for (int k0 = 0; k0 < K; k0 += 32) {
     const int k = k0 + kq;
     const bool k_ok = k < K;
-    const bf16x8 xf = grouped_frag(xr + k, k_ok && row >= 0);
+    bf16x8 xf[RT];
+#pragma unroll
+    for (int t = 0; t < RT; ++t) xf[t] = grouped_frag(xr[t] + k, k_ok && row[t] >= 0);
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
       const int o = o0 + c * 16 + r;
       const bool ok = k_ok && o < n_out;
-      acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(grouped_frag(wb + static_cast<int64_t>(o) * s.w_stride + k, ok), xf, acc[c], 0, 0, 0);
-      if constexpr (kEpilogue == kGrClampedGlu)
-        acc2[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(grouped_frag(wb2 + static_cast<int64_t>(o) * s.w_stride + k, ok), xf, acc2[c], 0, 0, 0);
+      const bf16x8 wf = grouped_frag(wb + static_cast<int64_t>(o) * s.w_stride + k, ok);
+#pragma unroll
+      for (int t = 0; t < RT; ++t) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[t], acc[t][c], 0, 0, 0);
+      if constexpr (kEpilogue == kGrClampedGlu) {
+        const bf16x8 wf2 = grouped_frag(wb2 + static_cast<int64_t>(o) * s.w_stride + k, ok);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc2[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2, xf[t], acc2[t][c], 0, 0, 0);
+      }
     }
   }
-  if (row < 0) return;
-  const int out_row = s.tiles_per_batch > 0 ? row : slot;
-  TO* dst = out + static_cast<int64_t>(out_row) * s.out_stride + batch * s.out_batch_step;
-  float weight = 1.f, lim = 0.f;
-  if constexpr (kEpilogue == kGrClampedGlu) {
-    weight = slot_weight ? slot_weight[slot] : 1.f;
-    lim = last ? s.limit_last : s.limit;
-  }
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
+  for (int t = 0; t < RT; ++t) {
+    if (row[t] < 0) continue;
+    const int slot = slot0 + t * 16 + r;
+    const int out_row = s.tiles_per_batch > 0 ? row[t] : slot;
+    TO* dst = out + static_cast<int64_t>(out_row) * s.out_stride + batch * s.out_batch_step;
+    float weight = 1.f, lim = 0.f;
+    if constexpr (kEpilogue == kGrClampedGlu) {
+      weight = slot_weight ? slot_weight[slot] : 1.f;
+      lim = last ? s.limit_last : s.limit;
+    }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int o = o0 + c * 16 + (lane / 16) * 4 + i;
-      if (o >= n_out) continue;
-      float y = acc[c][i];
-      if constexpr (kEpilogue == kGrSigmoidGate) {
-        const float g = bf16_to_f32(gate[static_cast<int64_t>(out_row) * s.gate_stride + batch * s.out_batch_step + o]);
-        y *= 1.f / (1.f + __expf(-g));
-      } else if constexpr (kEpilogue == kGrClampedGlu) {
-        const float a = fminf(y, lim);
-        const float b = fminf(fmaxf(acc2[c][i], -lim), lim);
-        y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
+    for (int c = 0; c < NC; ++c) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = o0 + c * 16 + (lane / 16) * 4 + i;
+        if (o >= n_out) continue;
+        float y = acc[t][c][i];
+        if constexpr (kEpilogue == kGrSigmoidGate) {
+          const float g = bf16_to_f32(gate[static_cast<int64_t>(out_row) * s.gate_stride + batch * s.out_batch_step + o]);
+          y *= 1.f / (1.f + __expf(-g));
+        } else if constexpr (kEpilogue == kGrClampedGlu) {
+          const float a = fminf(y, lim);
+          const float b = fminf(fmaxf(acc2[t][c][i], -lim), lim);
+          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
+        }
+        store_f32(dst + o, y);
       }
-      store_f32(dst + o, y);
     }
   }
 }
 
 // ---- the rows of every expert, side by side ------------------------------------------------------------------
 // chosen, weights [T, top]: the experts a row takes and its weights. Slots: every expert's rows together, an
-// expert's share padded to a multiple of 16, in expert order; then (with `shared`) all T rows once more for the
+// expert's share padded to a multiple of `pad` (a tile's rows: 16 or 64), in expert order; then (with `shared`) all T rows once more for the
 // expert every row takes, as batch E. Outputs: row_in[slot] (the row, or -1), slot_weight[slot], slot_of[t * top + k]
 // (where row t's k-th choice went) and slot_of[T * top + t] (its slot of the shared expert), tile_batch[tile] (the
-// expert of a tile of 16 slots, -1 beyond the last). Which slot of its expert's share a row gets depends on the
+// expert of a tile of `pad` slots, -1 beyond the last). Which slot of its expert's share a row gets depends on the
 // order in which threads arrive, which changes no result: a slot's values depend on its row alone.
 // One block; experts up to 512.
 __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __restrict__ chosen, const float* __restrict__ weights, int32_t* __restrict__ row_in,
                                                            float* __restrict__ slot_weight, int32_t* __restrict__ slot_of, int32_t* __restrict__ tile_batch,
-                                                           int T, int top, int experts, int shared, int slots, int tiles) {
+                                                           int T, int top, int experts, int shared, int slots, int tiles, int pad) {
   __shared__ int count[512], first[513], cursor[512];
   for (int e = threadIdx.x; e < experts; e += 1024) count[e] = cursor[e] = 0;
   for (int i = threadIdx.x; i < slots; i += 1024) {
@@ -137,13 +159,13 @@ __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __rest
     int at = 0;
     for (int e = 0; e < experts; ++e) {
       first[e] = at;
-      at += (count[e] + 15) / 16 * 16;
+      at += (count[e] + pad - 1) / pad * pad;
     }
     first[experts] = at;
   }
   __syncthreads();
   for (int e = threadIdx.x; e < experts; e += 1024)
-    for (int t = first[e] / 16; t < first[e + 1] / 16; ++t) tile_batch[t] = e;
+    for (int t = first[e] / pad; t < first[e + 1] / pad; ++t) tile_batch[t] = e;
   for (int i = threadIdx.x; i < pairs; i += 1024) {
     const int e = chosen[i];
     const int slot = first[e] + atomicAdd(&cursor[e], 1);
@@ -158,7 +180,7 @@ __global__ void __launch_bounds__(1024) expert_rows_kernel(const int32_t* __rest
       slot_weight[base + t] = 1.f;
       slot_of[pairs + t] = base + t;
     }
-    for (int t = threadIdx.x; t < (T + 15) / 16; t += 1024) tile_batch[base / 16 + t] = experts;
+    for (int t = threadIdx.x; t < (T + pad - 1) / pad; t += 1024) tile_batch[base / pad + t] = experts;
   }
 }
 
@@ -180,19 +202,21 @@ using namespace alofa;
 
 template <int kEpilogue, typename TO>
 static int launch_grouped(void* out, const void* x, const void* W, const void* W2, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
-                          const float* slot_weight, const GroupedShape& s, hipStream_t stream) {
+                          const float* slot_weight, const GroupedShape& s, int tile_rows, hipStream_t stream) {
   const int widest = s.n_out > s.n_out_last ? s.n_out : s.n_out_last;
   // narrower groups of columns where the tiles are too few to fill the chip
   const int64_t wide_tasks = static_cast<int64_t>(s.tiles) * ((widest + 63) / 64);
-  const int nc = wide_tasks >= 2 * compute_units() * 4 ? 4 : (wide_tasks * 2 >= 2 * compute_units() * 4 ? 2 : 1);
+  const int64_t fill = 2 * static_cast<int64_t>(compute_units()) * 4;
+  const int nc = (tile_rows == 64 || wide_tasks >= fill) ? 4 : (wide_tasks * 2 >= fill ? 2 : 1);
   const int col_groups = (widest + nc * 16 - 1) / (nc * 16);
   const int64_t tasks = static_cast<int64_t>(s.tiles) * col_groups;
   const unsigned grid = static_cast<unsigned>((tasks + 3) / 4);
-#define ALOFA_GROUPED(NC) grouped_product_kernel<NC, kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), \
+#define ALOFA_GROUPED(RT, NC) grouped_product_kernel<RT, NC, kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), \
     static_cast<const bf16_t*>(W2), tile_batch, row_in, static_cast<const bf16_t*>(gate), slot_weight, s, col_groups)
-  if (nc == 4) ALOFA_GROUPED(4);
-  else if (nc == 2) ALOFA_GROUPED(2);
-  else ALOFA_GROUPED(1);
+  if (tile_rows == 64) ALOFA_GROUPED(4, 4);
+  else if (nc == 4) ALOFA_GROUPED(1, 4);
+  else if (nc == 2) ALOFA_GROUPED(1, 2);
+  else ALOFA_GROUPED(1, 1);
 #undef ALOFA_GROUPED
   return check_launch("grouped_product");
 }
@@ -200,32 +224,34 @@ static int launch_grouped(void* out, const void* x, const void* W, const void* W
 // out dtype: kBF16 or kF32; x, W, W2, gate bfloat16. epilogue: 0 store, 1 times sigmoid(gate), 2 clamped GLU of (W, W2) times slot_weight.
 extern "C" int alofa_grouped_product(void* out, int out_dtype, int64_t out_stride, int64_t out_batch_step, const void* x, int64_t x_stride, int64_t x_batch_step,
                                      const void* W, const void* W2, int64_t w_stride, int64_t w_batch_step, int n_out, int K, int last_batch, int n_out_last,
-                                     int K_last, int rows, int x_by_slot, int tiles, int tiles_per_batch, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
+                                     int K_last, int rows, int x_by_slot, int tiles, int tiles_per_batch, int tile_rows, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
                                      int64_t gate_stride, const float* slot_weight, float limit, float limit_last, float slope, int epilogue, hipStream_t stream) {
   ALOFA_REQUIRE(n_out > 0 && K > 0 && rows >= 0 && tiles >= 0, "grouped_product: bad sizes (n_out=%d K=%d rows=%d tiles=%d)", n_out, K, rows, tiles);
   ALOFA_REQUIRE(K % 8 == 0 && K_last % 8 == 0 && x_stride % 8 == 0 && x_batch_step % 8 == 0 && w_stride % 8 == 0 && w_batch_step % 8 == 0 &&
                     reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(W) % 16 == 0 && (W2 == nullptr || reinterpret_cast<uintptr_t>(W2) % 16 == 0),
                 "grouped_product: operands must be 16-byte aligned along the reduction (K=%d x_stride=%lld w_stride=%lld)", K, (long long)x_stride, (long long)w_stride);
   ALOFA_REQUIRE((tiles_per_batch > 0) != (tile_batch != nullptr), "grouped_product: tiles are dense (tiles_per_batch) or listed (tile_batch)");
+  ALOFA_REQUIRE(tile_rows == 16 || tile_rows == 64, "grouped_product: tiles of 16 or 64 rows (tile_rows=%d)", tile_rows);
   ALOFA_REQUIRE(epilogue != kGrSigmoidGate || gate, "grouped_product: the gate epilogue needs gates");
   ALOFA_REQUIRE(epilogue != kGrClampedGlu || (W2 && out_dtype == kBF16), "grouped_product: the GLU epilogue needs a second matrix and writes bfloat16");
   if (rows == 0 || tiles == 0) return 0;
   GroupedShape s{out_stride, out_batch_step, x_stride, x_batch_step, w_stride, w_batch_step, n_out, K, last_batch, n_out_last, K_last, rows, x_by_slot, tiles, tiles_per_batch,
                  gate_stride, limit, limit_last, slope};
-  if (epilogue == kGrStore && out_dtype == kBF16) return launch_grouped<kGrStore, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, stream);
-  if (epilogue == kGrStore && out_dtype == kF32) return launch_grouped<kGrStore, float>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, stream);
-  if (epilogue == kGrSigmoidGate && out_dtype == kBF16) return launch_grouped<kGrSigmoidGate, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, stream);
-  if (epilogue == kGrClampedGlu) return launch_grouped<kGrClampedGlu, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, stream);
+  if (epilogue == kGrStore && out_dtype == kBF16) return launch_grouped<kGrStore, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
+  if (epilogue == kGrStore && out_dtype == kF32) return launch_grouped<kGrStore, float>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
+  if (epilogue == kGrSigmoidGate && out_dtype == kBF16) return launch_grouped<kGrSigmoidGate, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
+  if (epilogue == kGrClampedGlu) return launch_grouped<kGrClampedGlu, bf16_t>(out, x, W, W2, tile_batch, row_in, gate, slot_weight, s, tile_rows, stream);
   ALOFA_REQUIRE(false, "grouped_product: no such epilogue and output type (epilogue=%d out=%d)", epilogue, out_dtype);
   return 1;
 }
 
 extern "C" int alofa_expert_rows(const int32_t* chosen, const float* weights, int32_t* row_in, float* slot_weight, int32_t* slot_of, int32_t* tile_batch,
-                                 int T, int top, int experts, int shared, int slots, int tiles, hipStream_t stream) {
+                                 int T, int top, int experts, int shared, int slots, int tiles, int pad, hipStream_t stream) {
   ALOFA_REQUIRE(T > 0 && top > 0 && experts > 0 && experts <= 512 && top <= experts, "expert_rows: bad sizes (T=%d top=%d experts=%d)", T, top, experts);
-  const int64_t need = (static_cast<int64_t>(T) * top + 15) / 16 * 16 + 16 * static_cast<int64_t>(experts) + (shared ? (T + 15) / 16 * 16 : 0);
-  ALOFA_REQUIRE(slots >= need && tiles * 16 >= slots, "expert_rows: room for %lld slots is needed (slots=%d tiles=%d)", (long long)need, slots, tiles);
-  expert_rows_kernel<<<1, 1024, 0, stream>>>(chosen, weights, row_in, slot_weight, slot_of, tile_batch, T, top, experts, shared, slots, tiles);
+  ALOFA_REQUIRE(pad == 16 || pad == 64, "expert_rows: tiles of 16 or 64 rows (pad=%d)", pad);
+  const int64_t need = (static_cast<int64_t>(T) * top + pad - 1) / pad * pad + pad * static_cast<int64_t>(experts) + (shared ? (T + pad - 1) / pad * pad : 0);
+  ALOFA_REQUIRE(slots >= need && static_cast<int64_t>(tiles) * pad >= slots, "expert_rows: room for %lld slots is needed (slots=%d tiles=%d)", (long long)need, slots, tiles);
+  expert_rows_kernel<<<1, 1024, 0, stream>>>(chosen, weights, row_in, slot_weight, slot_of, tile_batch, T, top, experts, shared, slots, tiles, pad);
   return check_launch("expert_rows");
 }
 

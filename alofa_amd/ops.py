@@ -1245,14 +1245,15 @@ def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor
 
 
 GR_STORE, GR_SIGMOID_GATE, GR_CLAMPED_GLU = 0, 1, 2
+GROUPED_BIG_TILES = 256     # rows of a step from which the many-small-products kernel takes tiles of 64 rows instead of 16
 
 
 def _grouped(out, out_step, x, x_step, w, w2, w_stride, w_step, n_out, K, last, rows, x_by_slot, tiles, tiles_per_batch, tile_batch, row_in,
-             gate, slot_weight, limit, limit_last, slope, epilogue) -> None:
+             gate, slot_weight, limit, limit_last, slope, epilogue, tile_rows=16) -> None:
     last_batch, n_out_last, K_last = last if last is not None else (-1, n_out, K)
     _call("alofa_grouped_product", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _L(out_step), _ptr(x), _L(_rows("x", x)), _L(x_step),
           _ptr(w), _ptr(w2), _L(w_stride), _L(w_step), _I(n_out), _I(K), _I(last_batch), _I(n_out_last), _I(K_last), _I(rows), _I(int(x_by_slot)), _I(tiles),
-          _I(tiles_per_batch), _ptr(tile_batch), _ptr(row_in), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _ptr(slot_weight),
+          _I(tiles_per_batch), _I(tile_rows), _ptr(tile_batch), _ptr(row_in), _ptr(gate), _L(_rows("gate", gate) if gate is not None else 0), _ptr(slot_weight),
           _F(limit), _F(limit_last), _F(slope), _I(epilogue), _stream())
 
 
@@ -1274,9 +1275,10 @@ def head_project(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, exact: boo
             raise AlofaError("shape_mismatch", "one gate per output", f"gate={tuple(gate.shape)} out={tuple(out.shape)}")
     T = x.shape[0]
     if not exact and out.dtype is torch.bfloat16 and w.dtype is torch.bfloat16 and din % 8 == 0 and _aligned_rows(x) and w.data_ptr() % 16 == 0 and T > 0:
-        per = (T + 15) // 16
+        tile_rows = 64 if T >= GROUPED_BIG_TILES else 16      # (tiles of 64 rows, which use a fragment of the matrix four times, once there are rows for them)
+        per = (T + tile_rows - 1) // tile_rows
         _grouped(out, dout, x, din, w, None, din, dout * din, dout, din, None, T, False, H * per, per, None, None, gate, None, 0.0, 0.0, 0.0,
-                 GR_SIGMOID_GATE if gate is not None else GR_STORE)
+                 GR_SIGMOID_GATE if gate is not None else GR_STORE, tile_rows)
         return
     for a in range(H):
         gemm(out[:, a * dout:(a + 1) * dout], x[:, a * din:(a + 1) * din], w[a], exact=exact)
@@ -1291,8 +1293,10 @@ class ExpertRows:
 
     def __init__(self, T: int, top: int, experts: int, shared: bool, scratch):
         self.T, self.top, self.experts, self.shared = T, top, experts, shared
-        self.slots = (T * top + 15) // 16 * 16 + 16 * experts + ((T + 15) // 16 * 16 if shared else 0)
-        self.tiles = self.slots // 16
+        # an expert's rows fill whole tiles: of 64 rows where the experts get that many on average, else of 16
+        pad = self.tile_rows = 64 if T >= GROUPED_BIG_TILES and T * top >= 64 * experts else 16
+        self.slots = (T * top + pad - 1) // pad * pad + pad * experts + ((T + pad - 1) // pad * pad if shared else 0)
+        self.tiles = self.slots // pad
         self.row_in, self.slot_weight = scratch("expert_row_in", (self.slots,), torch.int32), scratch("expert_slot_weight", (self.slots,), torch.float32)
         self.slot_of, self.tile_batch = scratch("expert_slot_of", (T * (top + 1),), torch.int32), scratch("expert_tile_batch", (self.tiles,), torch.int32)
 
@@ -1302,7 +1306,7 @@ def expert_rows(rows: ExpertRows, chosen: torch.Tensor, weights: torch.Tensor) -
     if tuple(chosen.shape) != (rows.T, rows.top) or tuple(weights.shape) != (rows.T, rows.top):
         raise AlofaError("shape_mismatch", "one choice and one weight per row and place", f"chosen={tuple(chosen.shape)} weights={tuple(weights.shape)}")
     _call("alofa_expert_rows", _ptr(chosen), _ptr(weights), _ptr(rows.row_in), _ptr(rows.slot_weight), _ptr(rows.slot_of), _ptr(rows.tile_batch),
-          _I(rows.T), _I(rows.top), _I(rows.experts), _I(int(rows.shared)), _I(rows.slots), _I(rows.tiles), _stream())
+          _I(rows.T), _I(rows.top), _I(rows.experts), _I(int(rows.shared)), _I(rows.slots), _I(rows.tiles), _I(rows.tile_rows), _stream())
 
 
 def can_group_experts(x: torch.Tensor, w_gate: torch.Tensor, ff: int, shared_ff: int) -> bool:
@@ -1321,7 +1325,7 @@ def experts_gate_up(act: torch.Tensor, x: torch.Tensor, w_gate: torch.Tensor, w_
     if tuple(w_gate.shape) != (F, h) or tuple(w_up.shape) != (F, h) or act.shape[0] < rows.slots or act.shape[1] < max(ff, shared_ff) or x.shape[0] != rows.T:
         raise AlofaError("shape_mismatch", "the experts' matrices or the slots' rows do not fit", f"act={tuple(act.shape)} x={tuple(x.shape)} w_gate={tuple(w_gate.shape)} F={F}")
     _grouped(act, 0, x, 0, w_gate, w_up, h, ff * h, ff, h, (rows.experts, shared_ff, h) if rows.shared else None, rows.slots, False, rows.tiles, 0,
-             rows.tile_batch, rows.row_in, None, rows.slot_weight, limit, shared_limit, slope, GR_CLAMPED_GLU)
+             rows.tile_batch, rows.row_in, None, rows.slot_weight, limit, shared_limit, slope, GR_CLAMPED_GLU, rows.tile_rows)
 
 
 def experts_down(y: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, rows: ExpertRows, ff: int, shared_ff: int) -> None:
@@ -1332,7 +1336,7 @@ def experts_down(y: torch.Tensor, act: torch.Tensor, w_down: torch.Tensor, rows:
     if w_down.shape[1] != F or tuple(y.shape) != (rows.slots, h) or act.shape[0] < rows.slots or not _aligned_rows(act) or F % 8:
         raise AlofaError("shape_mismatch", "the experts' matrices or the slots' rows do not fit", f"y={tuple(y.shape)} act={tuple(act.shape)} w_down={tuple(w_down.shape)} F={F}")
     _grouped(y, 0, act, 0, w_down, None, F, ff, h, ff, (rows.experts, h, shared_ff) if rows.shared else None, rows.slots, True, rows.tiles, 0,
-             rows.tile_batch, rows.row_in, None, None, 0.0, 0.0, 0.0, GR_STORE)
+             rows.tile_batch, rows.row_in, None, None, 0.0, 0.0, 0.0, GR_STORE, rows.tile_rows)
 
 
 def experts_sum(residual: torch.Tensor, y: torch.Tensor, rows: ExpertRows, scale: Optional[torch.Tensor] = None) -> None:

@@ -114,9 +114,9 @@ def _padded_heads(t: torch.Tensor, heads: int, size: int, to: int, order=None) -
     rest = tuple(t.shape[1:])
     t = t.reshape(heads, size, *rest)
     if to > size:
-        t = torch.cat([t, torch.zeros((heads, to - size, *rest), dtype=t.dtype)], dim=1)
+        t = torch.cat([t, torch.zeros((heads, to - size, *rest), dtype=t.dtype, device=t.device)], dim=1)
     if order is not None:
-        t = t[:, torch.tensor(order, dtype=torch.long)]
+        t = t[:, torch.tensor(order, dtype=torch.long, device=t.device)]
     return t.reshape(heads * to, *rest).contiguous()
 
 

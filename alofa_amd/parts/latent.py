@@ -73,9 +73,9 @@ class LatentAttention(Mixer):
         if self.latent_heads:
             # per head [out, in]: a query into the latent's channels (Uk_a^T, [d, dk], zero rows beyond r) and a result out of them (Uv_a, [dv, d], zero columns beyond r)
             uk = weights[pre + n["up_k"]].reshape(H, dk, r).transpose(1, 2)
-            self.w_query = rt.matrix(torch.cat([uk, torch.zeros(H, d - r, dk, dtype=uk.dtype)], dim=1).contiguous())
+            self.w_query = rt.matrix(torch.cat([uk, torch.zeros(H, d - r, dk, dtype=uk.dtype, device=uk.device)], dim=1).contiguous())
             uv = weights[pre + n["up_v"]].reshape(H, dv, r)
-            self.w_result = rt.matrix(torch.cat([uv, torch.zeros(H, dv, d - r, dtype=uv.dtype)], dim=2).contiguous())
+            self.w_result = rt.matrix(torch.cat([uv, torch.zeros(H, dv, d - r, dtype=uv.dtype, device=uv.device)], dim=2).contiguous())
             self.kv_heads = 1
         else:
             # keys and values per head, every head widened to one size with zero rows (zero columns of the output matrix)

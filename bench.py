@@ -28,8 +28,8 @@ context of 4,096) through the same engine and print their own line;
 ``--config 1.5b``, ``3b`` and ``14b`` run the continuous batch at those sizes.
 ``--sweep batch`` and ``--sweep context`` take any of the configurations.
 
-``--design tugalix`` measures another design beside Qwen2 at equal sizes: prefill of one prompt and decode steps at
-batch 1, 8 and 64, at a few widths (``--sizes``), a line per point and model."""
+``--design tugalix`` and ``--design rerupel`` measure another design beside Qwen2 at equal sizes: prefill of one prompt and
+decode steps at batch 1, 8 and 64, at a few widths (``--sizes``), a line per point and model."""
 import argparse
 import json
 import statistics
@@ -511,23 +511,39 @@ def tugalix_sizes(width, heads, dim, ff, layers, vocab=32000):
     return tug, qwen
 
 
+def rerupel_sizes(width, heads, dim, ff, layers, vocab=32000):
+    """A Rerupel model of ``layers`` layers (the first with a dense feed-forward, the others with sixteen experts of which a
+    token takes four, and one that every token takes; latents of twice a head's size; all layers but the first in a loop that
+    is passed once), and the Qwen2 model of equal width, heads and layers whose feed-forward has as many channels as a
+    token's five experts together."""
+    expert = max(64, ff // 8 // 64 * 64)
+    mixer = {"heads": heads, "dim": dim, "vdim": dim, "kv_rank": 2 * dim, "scale": dim ** -0.5}
+    moe = {"kind": "moe", "router": {"experts": 16, "top": 4, "scale": 1.0}, "expert": {"ff": expert, "limit": 7.0}, "shared": {"ff": expert, "limit": 7.0}}
+    rer = {"architecture": "Rerupel", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "residual_mult": 1.0, "logit_softcap": 30.0,
+           "embedding": {"scale": 1.0, "bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}}, "loop": {"start": 1, "stop": layers, "times": 1},
+           "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": ff} if i == 0 else moe} for i in range(layers)]}
+    qwen = dict(family(layers, width, heads, max(1, heads // 4), 5 * expert, vocab, False), head_dim=dim)
+    return rer, qwen
+
+
+DESIGN_MODELS = {"tugalix": tugalix_sizes, "rerupel": rerupel_sizes}
 DESIGN_SIZES = {"256": (256, 4, 64, 1024, 4), "1k": (1024, 16, 64, 4096, 8), "2k": (2048, 16, 128, 8192, 8), "4k": (4096, 32, 128, 14336, 4)}
 DESIGN_DEFAULT = ("1k", "2k", "4k")      # ("256": a small one, for a quick look)
 
 
 def designs(args):
     """Prefill (one prompt of 2,048 tokens in one step) and decode steps (batch 1, 8 and 64 at a context of about 550) of
-    Tugalix beside Qwen2 at equal sizes, random weights: one line per point and model."""
+    another design beside Qwen2 at equal sizes, random weights: one line per point and model."""
     sizes = args.sizes.split(",") if args.sizes else list(DESIGN_DEFAULT)
     for size in sizes:
         if size not in DESIGN_SIZES:
             print(f"no such size: {size} (known: {','.join(DESIGN_SIZES)})")
             return 2
-        for name, cfg in zip(("tugalix", "qwen2"), tugalix_sizes(*DESIGN_SIZES[size])):
+        for name, cfg in zip((args.design, "qwen2"), DESIGN_MODELS[args.design](*DESIGN_SIZES[size])):
             if args.only and name != args.only:
                 continue
             cfg = dict(cfg, vocab_size=cfg.get("vocab_size", cfg.get("vocab")))      # (the points draw their tokens by this key)
-            model = device_model({k: v for k, v in cfg.items() if not (name == "tugalix" and k == "vocab_size")}, args.dtype, 20261126)
+            model = device_model({k: v for k, v in cfg.items() if not (name != "qwen2" and k == "vocab_size")}, args.dtype, 20261126)
             weights = model[1].weight_bytes()
             if not args.no_prefill:
                 pp = PrefillPoint(model, cfg, args.dtype, T=args.prompt_tokens)
@@ -562,9 +578,9 @@ def main():
     ap.add_argument("--serve", action="store_true", help="the continuous batch of 64 requests (prompts of 128..2,048 tokens, 256 new tokens, chunks of 512) at the sizes of --config")
     ap.add_argument("--batches", default=None, help="with --sweep batch: these batch sizes only (comma-separated), e.g. to profile one point")
     ap.add_argument("--sweep", choices=["batch", "context"], default=None, help="decode steps over batch sizes or over contexts, a line per point (the sizes of --config)")
-    ap.add_argument("--design", choices=["tugalix"], default=None, help="prefill and decode of this design beside Qwen2 at equal sizes (--sizes), a line per point")
+    ap.add_argument("--design", choices=sorted(DESIGN_MODELS), default=None, help="prefill and decode of this design beside Qwen2 at equal sizes (--sizes), a line per point")
     ap.add_argument("--sizes", default=None, help=f"with --design: which of {','.join(DESIGN_SIZES)} (comma-separated; default {','.join(DESIGN_DEFAULT)})")
-    ap.add_argument("--only", choices=["tugalix", "qwen2"], default=None, help="with --design: this model alone (for profiling)")
+    ap.add_argument("--only", choices=sorted(DESIGN_MODELS) + ["qwen2"], default=None, help="with --design: this model alone (for profiling)")
     ap.add_argument("--prompt-tokens", type=int, default=2048, help="with --design: tokens of the prefill point's prompt")
     ap.add_argument("--no-prefill", action="store_true", help="with --design: decode points only")
     args = ap.parse_args()

@@ -178,7 +178,7 @@ def test_routed_experts_as_one_product(dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("heads, din, dout, rows", [(6, 64, 64, 5), (3, 40, 16, 1), (5, 15, 9, 70), (20, 16, 64, 130), (2, 128, 256, 33)])
+@pytest.mark.parametrize("heads, din, dout, rows", [(6, 64, 64, 5), (3, 40, 16, 1), (5, 15, 9, 70), (20, 16, 64, 130), (2, 128, 256, 33), (4, 32, 48, 300), (3, 96, 40, 1000)])
 def test_a_projection_per_head(heads, din, dout, rows, dtype):
     from alofa_amd import ops
     rng = np.random.default_rng(heads)
@@ -192,7 +192,8 @@ def test_a_projection_per_head(heads, din, dout, rows, dtype):
     assert (got[:, :8] == 5.0).all()
 
 
-@pytest.mark.parametrize("T, h, E, top, ff, sff", [(21, 40, 5, 2, 16, 24), (1, 64, 8, 3, 96, 96), (150, 72, 16, 4, 8, 0), (64, 48, 4, 1, 40, 8), (5, 200, 3, 1, 24, 48)])
+@pytest.mark.parametrize("T, h, E, top, ff, sff", [(21, 40, 5, 2, 16, 24), (1, 64, 8, 3, 96, 96), (150, 72, 16, 4, 8, 0), (64, 48, 4, 1, 40, 8), (5, 200, 3, 1, 24, 48),
+                                                  (300, 64, 4, 2, 72, 40), (700, 40, 6, 3, 16, 0)])
 def test_routed_experts_slot_by_slot(T, h, E, top, ff, sff):
     """The rows sorted by expert and every expert against its own rows only, against the plain sum over the experts a token
     takes; every row lands in exactly one slot per choice."""
@@ -220,9 +221,9 @@ def test_routed_experts_slot_by_slot(T, h, E, top, ff, sff):
     for t in range(T):
         for k in range(top):
             slot = slot_of[t * top + k]
-            assert row_in[slot] == t and tile_batch[slot // 16] == picks[t, k]
+            assert row_in[slot] == t and tile_batch[slot // rows.tile_rows] == picks[t, k]
         if sff:
-            assert row_in[slot_of[T * top + t]] == t and tile_batch[slot_of[T * top + t] // 16] == E
+            assert row_in[slot_of[T * top + t]] == t and tile_batch[slot_of[T * top + t] // rows.tile_rows] == E
     assert (row_in >= 0).sum() == T * (top + (1 if sff else 0))
     act = torch.zeros(rows.slots, (max(ff, sff) + 7) // 8 * 8, dtype=bf, device=DEV)
     ops.experts_gate_up(act, x, w_gate, w_up, rows, ff, sff, 1.0, 0.6, 1.702)
