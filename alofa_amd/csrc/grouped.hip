@@ -33,20 +33,33 @@ struct GroupedShape {
   float limit, limit_last, slope;       // kGrClampedGlu
 };
 
-__device__ __forceinline__ bf16x8 grouped_frag(const bf16_t* __restrict__ p, bool ok) {
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if (ok) v = *reinterpret_cast<const uint4*>(p);
+// Every lane issues every load (from the operand's first bytes where its own are not wanted) and what is not wanted is cleared
+// afterwards: loads under a branch are waited for one by one, loads without one are in flight together.
+__device__ __forceinline__ uint4 grouped_load(const bf16_t* __restrict__ base, int64_t offset, bool ok) {
+  return *reinterpret_cast<const uint4*>(base + (ok ? offset : 0));
+}
+__device__ __forceinline__ bf16x8 grouped_frag(uint4 v, bool ok) {
+  if (!ok) v = make_uint4(0, 0, 0, 0);
   return __builtin_bit_cast(bf16x8, v);
 }
 
-template <int RT, int NC, int kEpilogue, typename TO>
+// RT: 16-row tiles a task takes together (a tile is then 16 * RT rows): a fragment of the matrix serves them all.
+// KW: wavefronts that share a task's reduction (1: a block runs four tasks, a wavefront each; 4: a block runs one task, wavefront w
+// takes the steps of 32 along K numbered w, w + 4, ..., and the four partial sums are added in LDS in the wavefronts' order: for
+// steps of few rows, where the tasks are few and a lone wavefront's chain of loads is what the launch waits for).
+// kAhead: steps of 32 along K whose loads are issued together.
+template <int RT, int NC, int KW, int kEpilogue, typename TO>
 __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
                                                               const bf16_t* __restrict__ W2, const int32_t* __restrict__ tile_batch,
                                                               const int32_t* __restrict__ row_in, const bf16_t* __restrict__ gate,
                                                               const float* __restrict__ slot_weight, GroupedShape s, int col_groups) {
-  // RT: 16-row tiles a wavefront takes together (a tile is then 16 * RT rows): a fragment of the matrix serves them all
+  constexpr bool kGlu = kEpilogue == kGrClampedGlu;
+  constexpr int kAhead = RT == 1 ? 4 : 2;
+  constexpr int kSums = kGlu ? 2 : 1;
+  __shared__ f32x4 red[KW == 1 ? 1 : 3][KW == 1 ? 1 : RT * NC * kSums][KW == 1 ? 1 : 64];
   const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
-  const int64_t task = static_cast<int64_t>(blockIdx.x) * 4 + wave;
+  const int64_t task = KW == 1 ? static_cast<int64_t>(blockIdx.x) * 4 + wave : blockIdx.x;
+  const int kw = KW == 1 ? 0 : wave;
   const int tile = static_cast<int>(task / col_groups), cg = static_cast<int>(task % col_groups);
   if (tile >= s.tiles) return;
   int batch, slot0;
@@ -64,42 +77,85 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
   if (o0 >= n_out) return;
   const int r = lane % 16, kq = (lane / 16) * 8;
   int row[RT];
-  const bf16_t* xr[RT];
+  int64_t x_at[RT];
   bool any = false;
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
     const int slot = slot0 + t * 16 + r;
     row[t] = -1;
     if (slot < s.rows) row[t] = row_in ? row_in[slot] : slot;
-    xr[t] = x + static_cast<int64_t>(row[t] < 0 ? 0 : (s.x_by_slot ? slot : row[t])) * s.x_stride + batch * s.x_batch_step;
+    x_at[t] = static_cast<int64_t>(row[t] < 0 ? 0 : (s.x_by_slot ? slot : row[t])) * s.x_stride + batch * s.x_batch_step;
     any = any || row[t] >= 0;
   }
-  if (!__any(any)) return;
-  const bf16_t* wb = W + batch * s.w_batch_step, *wb2 = kEpilogue == kGrClampedGlu ? W2 + batch * s.w_batch_step : nullptr;
+  if (!__any(any)) return;      // (the whole block alike when it shares a task: no barrier is left waiting)
+  const bf16_t* wb = W + batch * s.w_batch_step, *wb2 = kGlu ? W2 + batch * s.w_batch_step : nullptr;
+  int64_t w_at[NC];
+  bool o_ok[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int o = o0 + c * 16 + r;
+    o_ok[c] = o < n_out;
+    w_at[c] = static_cast<int64_t>(o_ok[c] ? o : 0) * s.w_stride;
+  }
   f32x4 acc[RT][NC], acc2[RT][NC];
 #pragma unroll
   for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int c = 0; c < NC; ++c) acc[t][c] = acc2[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
-  for (int k0 = 0; k0 < K; k0 += 32) {
-    const int k = k0 + kq;
-    const bool k_ok = k < K;
-    bf16x8 xf[RT];
+  for (int k0 = kw * 32; k0 < K; k0 += 32 * KW * kAhead) {
+    uint4 xv[kAhead][RT], wv[kAhead][NC], wv2[kAhead][kGlu ? NC : 1];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) xf[t] = grouped_frag(xr[t] + k, k_ok && row[t] >= 0);
+    for (int a = 0; a < kAhead; ++a) {
+      const int k = k0 + a * 32 * KW + kq;
+      const bool k_ok = k < K;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-      const int o = o0 + c * 16 + r;
-      const bool ok = k_ok && o < n_out;
-      const bf16x8 wf = grouped_frag(wb + static_cast<int64_t>(o) * s.w_stride + k, ok);
+      for (int t = 0; t < RT; ++t) xv[a][t] = grouped_load(x, x_at[t] + k, k_ok);
 #pragma unroll
-      for (int t = 0; t < RT; ++t) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[t], acc[t][c], 0, 0, 0);
-      if constexpr (kEpilogue == kGrClampedGlu) {
-        const bf16x8 wf2 = grouped_frag(wb2 + static_cast<int64_t>(o) * s.w_stride + k, ok);
-#pragma unroll
-        for (int t = 0; t < RT; ++t) acc2[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2, xf[t], acc2[t][c], 0, 0, 0);
+      for (int c = 0; c < NC; ++c) {
+        wv[a][c] = grouped_load(wb, w_at[c] + k, k_ok);
+        if constexpr (kGlu) wv2[a][c] = grouped_load(wb2, w_at[c] + k, k_ok);
       }
     }
+#pragma unroll
+    for (int a = 0; a < kAhead; ++a) {
+      const bool k_ok = k0 + a * 32 * KW + kq < K;
+      bf16x8 xf[RT];
+#pragma unroll
+      for (int t = 0; t < RT; ++t) xf[t] = grouped_frag(xv[a][t], k_ok && row[t] >= 0);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const bf16x8 wf = grouped_frag(wv[a][c], k_ok && o_ok[c]);
+#pragma unroll
+        for (int t = 0; t < RT; ++t) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[t], acc[t][c], 0, 0, 0);
+        if constexpr (kGlu) {
+          const bf16x8 wf2 = grouped_frag(wv2[a][c], k_ok && o_ok[c]);
+#pragma unroll
+          for (int t = 0; t < RT; ++t) acc2[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf2, xf[t], acc2[t][c], 0, 0, 0);
+        }
+      }
+    }
+  }
+  if constexpr (KW > 1) {      // the partial sums of wavefronts 1, 2, 3 join wavefront 0's, in that order
+    if (wave > 0) {
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          red[wave - 1][(t * NC + c) * kSums][lane] = acc[t][c];
+          if constexpr (kGlu) red[wave - 1][(t * NC + c) * kSums + 1][lane] = acc2[t][c];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int w = 0; w < 3; ++w)
+#pragma unroll
+      for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          acc[t][c] += red[w][(t * NC + c) * kSums][lane];
+          if constexpr (kGlu) acc2[t][c] += red[w][(t * NC + c) * kSums + 1][lane];
+        }
   }
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
@@ -108,7 +164,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
     const int out_row = s.tiles_per_batch > 0 ? row[t] : slot;
     TO* dst = out + static_cast<int64_t>(out_row) * s.out_stride + batch * s.out_batch_step;
     float weight = 1.f, lim = 0.f;
-    if constexpr (kEpilogue == kGrClampedGlu) {
+    if constexpr (kGlu) {
       weight = slot_weight ? slot_weight[slot] : 1.f;
       lim = last ? s.limit_last : s.limit;
     }
@@ -122,7 +178,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
         if constexpr (kEpilogue == kGrSigmoidGate) {
           const float g = bf16_to_f32(gate[static_cast<int64_t>(out_row) * s.gate_stride + batch * s.out_batch_step + o]);
           y *= 1.f / (1.f + __expf(-g));
-        } else if constexpr (kEpilogue == kGrClampedGlu) {
+        } else if constexpr (kGlu) {
           const float a = fminf(y, lim);
           const float b = fminf(fmaxf(acc2[t][c][i], -lim), lim);
           y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
@@ -204,19 +260,21 @@ template <int kEpilogue, typename TO>
 static int launch_grouped(void* out, const void* x, const void* W, const void* W2, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
                           const float* slot_weight, const GroupedShape& s, int tile_rows, hipStream_t stream) {
   const int widest = s.n_out > s.n_out_last ? s.n_out : s.n_out_last;
-  // narrower groups of columns where the tiles are too few to fill the chip
+  // Tiles of 64 rows: a wavefront a task of 64 columns. Tiles of 16 rows: while the tasks of 64 columns are too few to give every
+  // SIMD of the chip two wavefronts, a block a task of 32 or 16 columns, its four wavefronts sharing the reduction.
   const int64_t wide_tasks = static_cast<int64_t>(s.tiles) * ((widest + 63) / 64);
   const int64_t fill = 2 * static_cast<int64_t>(compute_units()) * 4;
-  const int nc = (tile_rows == 64 || wide_tasks >= fill) ? 4 : (wide_tasks * 2 >= fill ? 2 : 1);
+  const bool shared_k = tile_rows == 16 && wide_tasks < fill;
+  const int nc = !shared_k ? 4 : (wide_tasks * 4 >= fill ? 2 : 1);
   const int col_groups = (widest + nc * 16 - 1) / (nc * 16);
   const int64_t tasks = static_cast<int64_t>(s.tiles) * col_groups;
-  const unsigned grid = static_cast<unsigned>((tasks + 3) / 4);
-#define ALOFA_GROUPED(RT, NC) grouped_product_kernel<RT, NC, kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), \
+  const unsigned grid = static_cast<unsigned>(shared_k ? tasks : (tasks + 3) / 4);
+#define ALOFA_GROUPED(RT, NC, KW) grouped_product_kernel<RT, NC, KW, kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), \
     static_cast<const bf16_t*>(W2), tile_batch, row_in, static_cast<const bf16_t*>(gate), slot_weight, s, col_groups)
-  if (tile_rows == 64) ALOFA_GROUPED(4, 4);
-  else if (nc == 4) ALOFA_GROUPED(1, 4);
-  else if (nc == 2) ALOFA_GROUPED(1, 2);
-  else ALOFA_GROUPED(1, 1);
+  if (tile_rows == 64) ALOFA_GROUPED(4, 4, 1);
+  else if (!shared_k) ALOFA_GROUPED(1, 4, 1);
+  else if (nc == 2) ALOFA_GROUPED(1, 2, 4);
+  else ALOFA_GROUPED(1, 1, 4);
 #undef ALOFA_GROUPED
   return check_launch("grouped_product");
 }
