@@ -277,20 +277,20 @@ __global__ void __launch_bounds__(256) concat_rows_kernel(TO* __restrict__ out, 
 // ---- RMSNorm of short rows, left several times side by side ------------------------------------------------
 // y = x / sqrt(mean(x^2) + eps) * w of `width` values; out[t, k * pad + j] = y[j] for k < copies, zeros for
 // width <= j < pad. One wavefront per row.
-template <typename TO, typename Acc>
-__global__ void __launch_bounds__(256) rmsnorm_spread_kernel(TO* __restrict__ out, int64_t out_stride, const float* __restrict__ x, int64_t x_stride,
+template <typename TO, typename Acc, typename TI = float>
+__global__ void __launch_bounds__(256) rmsnorm_spread_kernel(TO* __restrict__ out, int64_t out_stride, const TI* __restrict__ x, int64_t x_stride,
                                                              const float* __restrict__ w, int rows, int width, int pad, int copies, float eps) {
   const int t = blockIdx.x * 4 + threadIdx.x / kWave;
   if (t >= rows) return;
   const int lane = threadIdx.x % kWave;
-  const float* src = x + static_cast<int64_t>(t) * x_stride;
+  const TI* src = x + static_cast<int64_t>(t) * x_stride;
   Acc ss = 0;
-  for (int j = lane; j < width; j += kWave) ss += static_cast<Acc>(src[j]) * static_cast<Acc>(src[j]);
+  for (int j = lane; j < width; j += kWave) ss += static_cast<Acc>(load_f32(src + j)) * static_cast<Acc>(load_f32(src + j));
   ss = wave_sum(ss);
   const Acc inv = static_cast<Acc>(1) / sqrt(ss / static_cast<Acc>(width) + static_cast<Acc>(eps));
   TO* dst = out + static_cast<int64_t>(t) * out_stride;
   for (int j = lane; j < pad; j += kWave) {
-    const float y = j < width ? static_cast<float>(static_cast<Acc>(src[j]) * inv * static_cast<Acc>(w[j])) : 0.f;
+    const float y = j < width ? static_cast<float>(static_cast<Acc>(load_f32(src + j)) * inv * static_cast<Acc>(w[j])) : 0.f;
     for (int k = 0; k < copies; ++k) store_f32(dst + static_cast<int64_t>(k) * pad + j, y);
   }
 }
@@ -314,6 +314,41 @@ __global__ void __launch_bounds__(256) add_channel_scaled_kernel(float* __restri
   const int64_t e = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
   if (e >= elements) return;
   residual[e] = static_cast<float>(static_cast<Acc>(residual[e]) + static_cast<Acc>(scale[e % width]) * static_cast<Acc>(x[e]));
+}
+
+// ---- residual[t, :] += scale * x[t, :], and normed[t, :] = rmsnorm(residual[t, :]) * w: the sum into the stream and the norm the
+// next sub-layer starts with in one pass over the row (a block per row; the row's new values wait in registers) ----
+template <typename TO, typename Acc>
+__global__ void __launch_bounds__(256) add_channel_scaled_norm_kernel(float* __restrict__ residual, const float* __restrict__ x, const float* __restrict__ scale,
+                                                                      TO* __restrict__ normed, const float* __restrict__ w, int width, float eps) {
+  __shared__ Acc scratch[4];
+  constexpr int kOwn = 8;      // values a thread keeps (rows up to 2,048 wide; wider ones are read again)
+  const int64_t at = static_cast<int64_t>(blockIdx.x) * width;
+  float own[kOwn];
+  Acc ss = 0;
+#pragma unroll
+  for (int i = 0; i < kOwn; ++i) {
+    const int c = threadIdx.x + i * 256;
+    own[i] = 0.f;
+    if (c < width) {
+      own[i] = static_cast<float>(static_cast<Acc>(residual[at + c]) + static_cast<Acc>(scale[c]) * static_cast<Acc>(x[at + c]));
+      residual[at + c] = own[i];
+      ss += static_cast<Acc>(own[i]) * static_cast<Acc>(own[i]);
+    }
+  }
+  for (int c = threadIdx.x + kOwn * 256; c < width; c += 256) {
+    const float v = static_cast<float>(static_cast<Acc>(residual[at + c]) + static_cast<Acc>(scale[c]) * static_cast<Acc>(x[at + c]));
+    residual[at + c] = v;
+    ss += static_cast<Acc>(v) * static_cast<Acc>(v);
+  }
+  const Acc inv = static_cast<Acc>(1) / sqrt(block_sum<Acc, 256>(ss, scratch) / static_cast<Acc>(width) + static_cast<Acc>(eps));
+#pragma unroll
+  for (int i = 0; i < kOwn; ++i) {
+    const int c = threadIdx.x + i * 256;
+    if (c < width) store_f32(normed + at + c, static_cast<float>(static_cast<Acc>(own[i]) * inv * static_cast<Acc>(w[c])));
+  }
+  for (int c = threadIdx.x + kOwn * 256; c < width; c += 256)
+    store_f32(normed + at + c, static_cast<float>(static_cast<Acc>(residual[at + c]) * inv * static_cast<Acc>(w[c])));
 }
 
 // ---- x = cap * tanh(x / cap) ---------------------------------------------------------------------------------------
@@ -362,14 +397,17 @@ extern "C" int alofa_concat_rows(void* out, int out_dtype, const float* a, const
   return check_launch("concat_rows");
 }
 
-extern "C" int alofa_rmsnorm_spread(void* out, int out_dtype, int64_t out_stride, const float* x, int64_t x_stride, const float* w, int rows, int width, int pad,
+extern "C" int alofa_rmsnorm_spread(void* out, int out_dtype, int64_t out_stride, const void* xv, int x_dtype, int64_t x_stride, const float* w, int rows, int width, int pad,
                                     int copies, float eps, int exact, hipStream_t stream) {
+  const float* x = static_cast<const float*>(xv);
+  ALOFA_REQUIRE(x_dtype == kF32 || (x_dtype == kBF16 && out_dtype == kBF16 && !exact), "rmsnorm_spread: rows are float32, or bfloat16 with a bfloat16 result");
   ALOFA_REQUIRE(rows >= 0 && width > 0 && pad >= width && copies >= 1 && eps > 0.f && out_stride >= static_cast<int64_t>(copies) * pad && x_stride >= width,
                 "rmsnorm_spread: bad sizes (rows=%d width=%d pad=%d copies=%d)", rows, width, pad, copies);
   ALOFA_REQUIRE(!exact || out_dtype == kF32, "rmsnorm_spread: the exact path writes float32");
   if (rows == 0) return 0;
   const unsigned grid = static_cast<unsigned>((rows + 3) / 4);
-  if (exact) rmsnorm_spread_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
+  if (x_dtype == kBF16) rmsnorm_spread_kernel<bf16_t, float, bf16_t><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, static_cast<const bf16_t*>(xv), x_stride, w, rows, width, pad, copies, eps);
+  else if (exact) rmsnorm_spread_kernel<float, double><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
   else if (out_dtype == kF32) rmsnorm_spread_kernel<float, float><<<grid, 256, 0, stream>>>(static_cast<float*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
   else rmsnorm_spread_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(static_cast<bf16_t*>(out), out_stride, x, x_stride, w, rows, width, pad, copies, eps);
   return check_launch("rmsnorm_spread");
@@ -392,6 +430,18 @@ extern "C" int alofa_add_channel_scaled(float* residual, const float* x, const f
   if (exact) add_channel_scaled_kernel<double><<<blocks_of(rows * width), 256, 0, stream>>>(residual, x, scale, rows * width, width);
   else add_channel_scaled_kernel<float><<<blocks_of(rows * width), 256, 0, stream>>>(residual, x, scale, rows * width, width);
   return check_launch("add_channel_scaled");
+}
+
+extern "C" int alofa_add_channel_scaled_norm(float* residual, const float* x, const float* scale, void* normed, int normed_dtype, const float* w, int64_t rows,
+                                             int width, float eps, int exact, hipStream_t stream) {
+  ALOFA_REQUIRE(rows >= 0 && width > 0 && scale && normed && w && eps > 0.f, "add_channel_scaled_norm: bad arguments");
+  ALOFA_REQUIRE(!exact || normed_dtype == kF32, "add_channel_scaled_norm: the exact path writes float32");
+  if (rows == 0) return 0;
+  const unsigned grid = static_cast<unsigned>(rows);
+  if (exact) add_channel_scaled_norm_kernel<float, double><<<grid, 256, 0, stream>>>(residual, x, scale, static_cast<float*>(normed), w, width, eps);
+  else if (normed_dtype == kF32) add_channel_scaled_norm_kernel<float, float><<<grid, 256, 0, stream>>>(residual, x, scale, static_cast<float*>(normed), w, width, eps);
+  else add_channel_scaled_norm_kernel<bf16_t, float><<<grid, 256, 0, stream>>>(residual, x, scale, static_cast<bf16_t*>(normed), w, width, eps);
+  return check_launch("add_channel_scaled_norm");
 }
 
 extern "C" int alofa_softcap(float* x, float cap, int64_t elements, int exact, hipStream_t stream) {

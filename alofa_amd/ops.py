@@ -1162,13 +1162,15 @@ def concat_rows(out: torch.Tensor, a: torch.Tensor, b: torch.Tensor) -> None:
 
 
 def rmsnorm_spread(out: torch.Tensor, x: torch.Tensor, w: torch.Tensor, eps: float, pad: int, copies: int, exact: bool = False) -> None:
-    """out[t, k * pad + j] = rmsnorm(x[t])[j] * w[j] for k < copies (zeros for j from x's width up to pad). x float32 rows,
-    out rows of at least copies * pad values; row strides allowed."""
-    _gpu("out", out, None, 2), _gpu("x", x, torch.float32, 2), _gpu("w", w, torch.float32, 1), _contig("w", w)
+    """out[t, k * pad + j] = rmsnorm(x[t])[j] * w[j] for k < copies (zeros for j from x's width up to pad). x float32 rows (or
+    bfloat16 ones for a bfloat16 result), out rows of at least copies * pad values; row strides allowed."""
+    _gpu("out", out, None, 2), _gpu("x", x, None, 2), _gpu("w", w, torch.float32, 1), _contig("w", w)
+    if x.dtype is not torch.float32 and (x.dtype is not out.dtype or exact):
+        raise AlofaError("invalid_argument", "the rows to norm are float32, or bfloat16 for a bfloat16 result", f"x={x.dtype} out={out.dtype}")
     n, r = x.shape
     if out.shape[0] != n or out.shape[1] != copies * pad or w.shape[0] != r or pad < r:
         raise AlofaError("shape_mismatch", "the copies of the normed rows do not fit", f"out={tuple(out.shape)} x={tuple(x.shape)} pad={pad} copies={copies}")
-    _call("alofa_rmsnorm_spread", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(x), _L(_rows("x", x)), _ptr(w), _I(n), _I(r), _I(pad), _I(copies),
+    _call("alofa_rmsnorm_spread", _ptr(out), _I(dtype_code(out)), _L(_rows("out", out)), _ptr(x), _I(dtype_code(x)), _L(_rows("x", x)), _ptr(w), _I(n), _I(r), _I(pad), _I(copies),
           _F(eps), _I(int(exact)), _stream())
 
 
@@ -1238,10 +1240,29 @@ def clamped_glu(act: torch.Tensor, g: torch.Tensor, u: torch.Tensor, dense: Opti
           _F(limit), _F(shared_limit), _F(slope), _I(int(exact)), _stream())
 
 
-def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, scale: torch.Tensor, tmp: torch.Tensor, exact: bool = False) -> None:
-    """residual[t, c] += scale[c] * (a @ w.T)[t, c]; ``tmp`` float32 of the residual's shape takes the product on its way."""
+def gemm_channel_scaled(residual: torch.Tensor, a: torch.Tensor, w: torch.Tensor, scale: torch.Tensor, tmp: torch.Tensor, exact: bool = False,
+                        then_norm: Optional[tuple] = None) -> None:
+    """residual[t, c] += scale[c] * (a @ w.T)[t, c]; ``tmp`` float32 of the residual's shape takes the product on its way.
+    ``then_norm`` = (weight, eps, rows): afterwards ``rows`` holds the RMSNorm of the residual's new rows (the same launch adds and norms)."""
     gemm(tmp, a, w, exact=exact)
-    add_channel_scaled(residual, tmp, scale, exact)
+    if then_norm is None:
+        add_channel_scaled(residual, tmp, scale, exact)
+    else:
+        add_channel_scaled_norm(residual, tmp, scale, *then_norm, exact=exact)
+
+
+def add_channel_scaled_norm(residual: torch.Tensor, x: torch.Tensor, scale: torch.Tensor, weight: torch.Tensor, eps: float, normed: torch.Tensor,
+                            exact: bool = False) -> None:
+    """residual[t, c] += scale[c] * x[t, c]; normed[t] = rmsnorm(residual[t]) * weight."""
+    _gpu("residual", residual, torch.float32, 2), _gpu("x", x, torch.float32, 2), _gpu("scale", scale, torch.float32, 1), _gpu("weight", weight, torch.float32, 1)
+    _gpu("normed", normed, None, 2)
+    for n, t in (("residual", residual), ("x", x), ("scale", scale), ("weight", weight), ("normed", normed)):
+        _contig(n, t)
+    T, h = residual.shape
+    if x.shape != residual.shape or normed.shape != residual.shape or scale.shape[0] != h or weight.shape[0] != h:
+        raise AlofaError("shape_mismatch", "one factor and one norm weight per channel; rows of the stream's shape", f"residual={tuple(residual.shape)} x={tuple(x.shape)} normed={tuple(normed.shape)}")
+    _call("alofa_add_channel_scaled_norm", _ptr(residual), _ptr(x), _ptr(scale), _ptr(normed), _I(dtype_code(normed)), _ptr(weight), _L(T), _I(h), _F(eps),
+          _I(int(exact)), _stream())
 
 
 GR_STORE, GR_SIGMOID_GATE, GR_CLAMPED_GLU = 0, 1, 2

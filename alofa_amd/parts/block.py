@@ -12,6 +12,8 @@ filtered_prenorm: the same as prenorm with a filter over time in front of every 
 optional weighted average over the outputs of all layers so far."""
 from __future__ import annotations
 
+import os
+
 import torch
 
 from .. import ops
@@ -196,22 +198,41 @@ class ScaledPreNormBlock(Block):
     def mixers(self):
         return self.mixer.stateful_parts()
 
-    def _add(self, ctx, part, hidden, scale, *args):
+    def _sub_layer(self, ctx, part, norm, scale, hidden, buf, where=(), normed=False, then=None):
+        """hidden += scale * part(norm(hidden)). ``normed``: ``buf`` holds norm(hidden) already. ``then`` = (weight, eps, rows): the RMSNorm of
+        the new stream is left in ``rows`` on the way. A norm rides on the part's first product where the part says it can."""
+        rows = hidden.shape[0]
         if getattr(part, "takes_channel_scale", False):
-            part.forward(ctx, *args, hidden, scale=scale)
-        else:
-            apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
-            part.forward(ctx, *args, hidden, out=apart)
+            more = {"then": then} if then is not None else {}
+            if not normed and part.fuses_norm(norm, rows):
+                part.forward(ctx, *where, None, hidden, scale=scale, norm=norm, **more)
+            else:
+                if not normed:
+                    norm.forward(buf, hidden)
+                part.forward(ctx, *where, buf, hidden, scale=scale, **more)
+            return
+        if not normed:
+            norm.forward(buf, hidden)
+        apart = ctx.scratch("sub_out", tuple(hidden.shape), torch.float32)
+        part.forward(ctx, *where, buf, hidden, out=apart)
+        if then is None:
             ops.add_channel_scaled(hidden, apart, scale, self.rt.exact)
+        else:
+            ops.add_channel_scaled_norm(hidden, apart, scale, *then, exact=self.rt.exact)
 
     def forward(self, ctx, entry, hidden):
         buf = ctx.scratch("normed", tuple(hidden.shape), self.rt.dtype)
-        self.norms[0].forward(buf, hidden)
-        self._add(ctx, self.mixer, hidden, self.scales[0], (entry, 0), buf)
-        if self.feed_forward is not None:
-            self.norms[1].forward(buf, hidden)
-            self._add(ctx, self.feed_forward, hidden, self.scales[1], buf)
+        ff = self.feed_forward
+        then = None
+        if ff is not None and FUSE_SUMS and self.norms[1].as_rmsnorm() is not None and not (getattr(ff, "takes_channel_scale", False) and ff.fuses_norm(self.norms[1], hidden.shape[0])):
+            # the norm in front of the feed-forward is made by the launch that adds the mixer's result to the stream
+            then = (*self.norms[1].as_rmsnorm(), buf)
+        self._sub_layer(ctx, self.mixer, self.norms[0], self.scales[0], hidden, buf, where=((entry, 0),), then=then)
+        if ff is not None:
+            self._sub_layer(ctx, ff, self.norms[1], self.scales[1], hidden, buf, normed=then is not None)
 
+
+FUSE_SUMS = os.environ.get("ALOFA_FUSE_SUMS", "1") != "0"      # 0 (for measurements): a scaled sum into the stream and the norm behind it are two launches
 
 register_part("block", "prenorm", PreNormBlock)
 register_part("block", "scaled_prenorm", ScaledPreNormBlock)

@@ -94,9 +94,15 @@ class DenseActivated(FeedForward):
             pq = weights[pre + names["act"]].double().tolist()
             self.a, self.b = _softplus(pq[0]), 0.5 + _softplus(pq[1])
 
-    def forward(self, ctx, x, residual, scale=None):
+    def fuses_norm(self, norm, rows):
+        return not self.rt.exact and norm.as_rmsnorm() is not None and ops.can_fuse_norm(rows, self.w_up, self.rt.dtype)
+
+    def forward(self, ctx, x, residual, scale=None, norm=None):
         act = ctx.scratch("ff_act", (residual.shape[0], self.intermediate), self.rt.dtype)
-        ops.gemm(act, x, self.w_up, exact=self.rt.exact)
+        if norm is not None:      # the norm in front rides on the product
+            ops.gemm(act, residual, self.w_up, norm=norm.as_rmsnorm())
+        else:
+            ops.gemm(act, x, self.w_up, exact=self.rt.exact)
         if self.activation == "xielu":
             ops.activation(act, act, ops.XIELU, self.a, self.b, self.rt.exact)
         else:

@@ -91,8 +91,9 @@ class LatentAttention(Mixer):
         self.d = d
         self.w_q = rt.matrix(w_q)
         self.w_gate = rt.matrix(w_g) if self.gated else None
-        if self.gated and self.latent_heads and w_q.dtype is w_g.dtype:      # queries and gates in one product
-            self.w_in = rt.matrix(torch.cat([w_q, w_g], dim=0))
+        w_d = weights[pre + n["down"]]
+        if self.latent_heads and w_q.dtype is w_d.dtype and (not self.gated or w_g.dtype is w_q.dtype):      # queries, gates and the latent in one product
+            self.w_in = rt.matrix(torch.cat([w_q] + ([w_g] if self.gated else []) + [w_d], dim=0))
         else:
             self.w_in = None
         self.w_o = rt.matrix(w_o)
@@ -104,21 +105,32 @@ class LatentAttention(Mixer):
     def prepare(self, n_positions):
         self.position.table(n_positions)
 
-    def _latent(self, ctx, x, out, pad, copies):
+    def _latent(self, ctx, x, out, pad, copies, down=None):
         """The step's latents, normed, ``copies`` times side by side in ``out`` (each widened to ``pad`` channels with zeros)."""
-        down = ctx.scratch("latent_down", (x.shape[0], self.r), torch.float32)
-        ops.gemm(down, x, self.w_down, exact=self.rt.exact)
+        if down is None:
+            down = ctx.scratch("latent_down", (x.shape[0], self.r), torch.float32)
+            ops.gemm(down, x, self.w_down, exact=self.rt.exact)
         w, eps = self.norm
         ops.rmsnorm_spread(out, down, w, eps, pad, copies, self.rt.exact)
 
-    def forward(self, ctx, where, x, residual, scale=None, out=None):
+    def fuses_norm(self, norm, rows):
+        return (self.w_in is not None and not self.rt.exact and norm.as_rmsnorm() is not None and ops.can_fuse_norm(rows, self.w_in, self.rt.dtype))
+
+    def forward(self, ctx, where, x, residual, scale=None, out=None, norm=None, then=None):
+        """``norm``: x is None and the mixer's input is this norm of the residual's rows, applied by the first product. ``then`` =
+        (weight, eps, rows): the RMSNorm of the residual's new rows is left in ``rows`` (with ``scale``)."""
         T, exact, H, d = residual.shape[0], self.rt.exact, self.heads, self.d
         attn = ctx.scratch("attn", (T, H * d), self.rt.dtype)
+        down = None
         if self.latent_heads:
             if self.w_in is not None:
                 qg = ctx.scratch("latent_in", (T, self.w_in.shape[0]), self.rt.dtype)
-                ops.gemm(qg, x, self.w_in, exact=exact)
-                q, gate = qg[:, :H * self.dk], qg[:, H * self.dk:]
+                if norm is not None:
+                    ops.gemm(qg, residual, self.w_in, norm=norm.as_rmsnorm())
+                else:
+                    ops.gemm(qg, x, self.w_in, exact=exact)
+                q, gate = qg[:, :H * self.dk], (qg[:, H * self.dk:H * (self.dk + self.dv)] if self.gated else None)
+                down = qg[:, qg.shape[1] - self.r:]
             else:
                 q, gate = ctx.scratch("latent_q", (T, H * self.dk), self.rt.dtype), None
                 ops.gemm(q, x, self.w_q, exact=exact)
@@ -127,7 +139,7 @@ class LatentAttention(Mixer):
                     ops.gemm(gate, x, self.w_gate, exact=exact)
             # [a query per head | the latent as key | the latent as value]
             qkv = ctx.scratch("qkv", (T, (H + 2) * d), self.rt.dtype)
-            self._latent(ctx, x, qkv[:, H * d:], d, 2)
+            self._latent(ctx, x, qkv[:, H * d:], d, 2, down)
             ops.head_project(qkv[:, :H * d], q, self.w_query, exact)
             paged_attend(ctx, where, qkv, attn, H, 1, d, self.window, self.scale, self.position, self.rt)
             heads_out = ctx.scratch("latent_out", (T, H * self.dv), self.rt.dtype)
@@ -149,7 +161,7 @@ class LatentAttention(Mixer):
         elif scale is None:
             ops.gemm(residual, heads_out, self.w_o, add_to_out=True, exact=exact)
         else:
-            ops.gemm_channel_scaled(residual, heads_out, self.w_o, scale, ctx.scratch("sub_out", tuple(residual.shape), torch.float32), exact)
+            ops.gemm_channel_scaled(residual, heads_out, self.w_o, scale, ctx.scratch("sub_out", tuple(residual.shape), torch.float32), exact, then_norm=then)
 
 
 register_part("mixer", "latent_attention", LatentAttention)
