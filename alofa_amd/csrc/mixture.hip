@@ -11,45 +11,69 @@ namespace alofa {
 // sigmoid(z), without its saturation), the lower index first among equals. Outputs:
 //   dense [T, E]: sigmoid(z) * scale at the chosen experts, 0 elsewhere (weights sum to one first when `renorm`);
 //   chosen [T, top], weights [T, top]: the same as lists, in order of falling score.
-// One thread per token; E up to kMaxExperts.
+// A wavefront per token: lane l holds the products l, l + 64, ... (E up to kMaxExperts); a pick is the best of the lanes'
+// own bests, found by exchanges between lanes (value falling, index rising).
 constexpr int kMaxExperts = 512;
 
 template <typename Acc>
-__global__ void __launch_bounds__(64) route_top_kernel(const float* __restrict__ z, float* __restrict__ dense, int32_t* __restrict__ chosen,
-                                                       float* __restrict__ weights, int tokens, int experts, int top, float scale, int renorm) {
-  const int t = blockIdx.x * 64 + threadIdx.x;
+__global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ z, float* __restrict__ dense, int32_t* __restrict__ chosen,
+                                                        float* __restrict__ weights, int tokens, int experts, int top, float scale, int renorm) {
+  constexpr int kOwn = kMaxExperts / kWave;
+  const int t = blockIdx.x * 4 + threadIdx.x / kWave, lane = threadIdx.x % kWave;
   if (t >= tokens) return;
   const float* row = z + static_cast<int64_t>(t) * experts;
   float* d = dense + static_cast<int64_t>(t) * experts;
-  for (int e = 0; e < experts; ++e) d[e] = 0.f;
+  float own[kOwn];
+  bool taken[kOwn];
+#pragma unroll
+  for (int i = 0; i < kOwn; ++i) {
+    const int e = lane + i * kWave;
+    own[i] = e < experts ? row[e] : 0.f;
+    taken[i] = e >= experts;
+    if (e < experts) d[e] = 0.f;
+  }
   Acc total = 0;
-  float last = 0.f;
-  int last_e = -1;
   for (int k = 0; k < top; ++k) {
-    // the largest score below (last, last_e) in the order (score falling, index rising)
-    int best = -1;
-    float best_z = 0.f;
-    for (int e = 0; e < experts; ++e) {
-      const float v = row[e];
-      const bool after = k == 0 || v < last || (v == last && e > last_e);
-      if (after && (best < 0 || v > best_z)) {
-        best = e;
-        best_z = v;
+    float best = 0.f;
+    int best_e = 1 << 30;
+#pragma unroll
+    for (int i = 0; i < kOwn; ++i) {
+      const int e = lane + i * kWave;
+      if (!taken[i] && (best_e == 1 << 30 || own[i] > best)) {      // (rising e within the lane: the first of equals stays)
+        best = own[i];
+        best_e = e;
       }
     }
-    last = best_z;
-    last_e = best;
-    const Acc s = static_cast<Acc>(1) / (static_cast<Acc>(1) + exp(-static_cast<Acc>(best_z)));
+#pragma unroll
+    for (int m = 1; m < kWave; m <<= 1) {
+      const float other = __shfl_xor(best, m);
+      const int other_e = __shfl_xor(best_e, m);
+      if (other_e != 1 << 30 && (best_e == 1 << 30 || other > best || (other == best && other_e < best_e))) {
+        best = other;
+        best_e = other_e;
+      }
+    }
+#pragma unroll
+    for (int i = 0; i < kOwn; ++i)
+      if (lane + i * kWave == best_e) taken[i] = true;
+    const Acc s = static_cast<Acc>(1) / (static_cast<Acc>(1) + exp(-static_cast<Acc>(best)));
     total += s;
-    chosen[static_cast<int64_t>(t) * top + k] = best;
-    weights[static_cast<int64_t>(t) * top + k] = static_cast<float>(s);
+    if (lane == 0) {
+      chosen[static_cast<int64_t>(t) * top + k] = best_e;
+      weights[static_cast<int64_t>(t) * top + k] = static_cast<float>(s);      // (made final below)
+    }
   }
-  for (int k = 0; k < top; ++k) {
-    Acc w = static_cast<Acc>(weights[static_cast<int64_t>(t) * top + k]);
-    if (renorm) w /= total;
-    const float f = static_cast<float>(w * static_cast<Acc>(scale));
-    weights[static_cast<int64_t>(t) * top + k] = f;
-    d[chosen[static_cast<int64_t>(t) * top + k]] = f;
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (lane == 0) {
+    for (int k = 0; k < top; ++k) {
+      Acc w = static_cast<Acc>(weights[static_cast<int64_t>(t) * top + k]);
+      if (renorm) w /= total;
+      const float f = static_cast<float>(w * static_cast<Acc>(scale));
+      weights[static_cast<int64_t>(t) * top + k] = f;
+      d[chosen[static_cast<int64_t>(t) * top + k]] = f;
+    }
   }
 }
 
@@ -88,9 +112,9 @@ extern "C" int alofa_route_top(const float* z, float* dense, int32_t* chosen, fl
                                int exact, hipStream_t stream) {
   ALOFA_REQUIRE(tokens >= 0 && experts > 0 && experts <= kMaxExperts && top > 0 && top <= experts, "route_top: bad sizes (tokens=%d experts=%d top=%d)", tokens, experts, top);
   if (tokens == 0) return 0;
-  const unsigned grid = static_cast<unsigned>((tokens + 63) / 64);
-  if (exact) route_top_kernel<double><<<grid, 64, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
-  else route_top_kernel<float><<<grid, 64, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
+  const unsigned grid = static_cast<unsigned>((tokens + 3) / 4);
+  if (exact) route_top_kernel<double><<<grid, 256, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
+  else route_top_kernel<float><<<grid, 256, 0, stream>>>(z, dense, chosen, weights, tokens, experts, top, scale, renorm);
   return check_launch("route_top");
 }
 
