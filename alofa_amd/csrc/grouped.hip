@@ -13,6 +13,8 @@
 // row_in[slot] names the input row (-1: nothing); the output row is the slot.
 #include "common.h"
 
+#include <stdlib.h>
+
 namespace alofa {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -189,6 +191,135 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(TO* __restrict__ o
   }
 }
 
+// ---- tiles of 64 rows through LDS ---------------------------------------------------------------------------
+// The same products for steps of many rows: a block owns a tile of 64 rows and 256 rows of the matrix (256 output columns, or,
+// for the GLU, 128 gate and 128 up rows of the same columns), a wavefront 64 x 64 of it. Slabs of 32 along K take turns in two
+// LDS buffers: while the block multiplies one, every thread has the next one's five 16-byte pieces on their way in registers. A
+// slab's row is 64 bytes, its four pieces permuted by (row >> 2) & 3, so that the sixteen rows a quarter of a wavefront reads
+// together fall on distinct banks. Fragments and sums are those of the kernel above (one accumulator an output, ascending k).
+template <int kEpilogue, typename TO>
+__global__ void __launch_bounds__(256) grouped_tiled_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ W,
+                                                            const bf16_t* __restrict__ W2, const int32_t* __restrict__ tile_batch,
+                                                            const int32_t* __restrict__ row_in, const bf16_t* __restrict__ gate,
+                                                            const float* __restrict__ slot_weight, GroupedShape s, int col_blocks) {
+  constexpr bool kGlu = kEpilogue == kGrClampedGlu;
+  constexpr int kCols = kGlu ? 128 : 256;      // output columns of a block
+  __shared__ __attribute__((aligned(16))) uint4 xs[2][64 * 4], ws[2][256 * 4];
+  const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+  const int tile = blockIdx.x / col_blocks, cb = blockIdx.x % col_blocks;
+  int batch, slot0;
+  if (s.tiles_per_batch > 0) {
+    batch = tile / s.tiles_per_batch;
+    slot0 = (tile % s.tiles_per_batch) * 64;
+  } else {
+    batch = tile_batch[tile];
+    slot0 = tile * 64;
+  }
+  if (batch < 0) return;
+  const bool last = batch == s.last_batch;
+  const int n_out = last ? s.n_out_last : s.n_out, K = last ? s.K_last : s.K;
+  const int o0 = cb * kCols;
+  if (o0 >= n_out) return;
+  // what this thread brings in of every slab: piece `pc` of row `lr` of the rows, and of four rows of the matrix
+  const int lr = threadIdx.x / 4, pc = threadIdx.x % 4;
+  const int my_slot = slot0 + lr;
+  int my_row = -1;
+  if (my_slot < s.rows) my_row = row_in ? row_in[my_slot] : my_slot;
+  const bf16_t* x_src = x + static_cast<int64_t>(my_row < 0 ? 0 : (s.x_by_slot ? my_slot : my_row)) * s.x_stride + batch * s.x_batch_step;
+  const bf16_t* w_src[4];
+  bool w_ok[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int wr = lr + 64 * j;      // row of the block's 256 staged matrix rows
+    const int o = o0 + (kGlu ? wr % 128 : wr);
+    w_ok[j] = o < n_out;
+    w_src[j] = ((kGlu && wr >= 128) ? W2 : W) + batch * s.w_batch_step + static_cast<int64_t>(w_ok[j] ? o : 0) * s.w_stride;
+  }
+  const int x_dst = lr * 4 + (pc ^ ((lr >> 2) & 3));
+  // this wavefront's four chunks of 16 staged matrix rows: its 64 columns, or its 32 gate columns and the same 32 up columns
+  int chunk_row[4];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) chunk_row[c] = kGlu ? (c < 2 ? wave * 32 + c * 16 : 128 + wave * 32 + (c - 2) * 16) : wave * 64 + c * 16;
+  const int r = lane % 16, q = lane / 16;
+  f32x4 acc[4][4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) acc[t][c] = f32x4{0.f, 0.f, 0.f, 0.f};
+  uint4 xv, wv[4];
+  auto fetch = [&](int k0) {
+    const bool k_ok = k0 + pc * 8 < K;
+    const int64_t k = k_ok ? k0 + pc * 8 : 0;      // (a piece past the end of K reads the row's first bytes and is cleared)
+    xv = *reinterpret_cast<const uint4*>(x_src + k);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wv[j] = *reinterpret_cast<const uint4*>(w_src[j] + k);
+    if (!k_ok || my_row < 0) xv = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (!k_ok || !w_ok[j]) wv[j] = make_uint4(0, 0, 0, 0);
+  };
+  auto stage = [&](int buf) {
+    xs[buf][x_dst] = xv;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) ws[buf][(lr + 64 * j) * 4 + (pc ^ ((lr >> 2) & 3))] = wv[j];      // ((lr + 64 j) >> 2) & 3 == (lr >> 2) & 3
+  };
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  const int slabs = (K + 31) / 32;
+  for (int sl = 0; sl < slabs; ++sl) {
+    const int buf = sl & 1;
+    if (sl + 1 < slabs) fetch((sl + 1) * 32);
+    bf16x8 xf[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+      const int row = t * 16 + r;
+      xf[t] = __builtin_bit_cast(bf16x8, xs[buf][row * 4 + (q ^ ((row >> 2) & 3))]);
+    }
+#pragma unroll
+    for (int c = 0; c < 4; ++c) {
+      const int row = chunk_row[c] + r;
+      const bf16x8 wf = __builtin_bit_cast(bf16x8, ws[buf][row * 4 + (q ^ ((row >> 2) & 3))]);
+#pragma unroll
+      for (int t = 0; t < 4; ++t) acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[t], acc[t][c], 0, 0, 0);
+    }
+    if (sl + 1 < slabs) stage(buf ^ 1);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int slot = slot0 + t * 16 + r;
+    int row = -1;
+    if (slot < s.rows) row = row_in ? row_in[slot] : slot;
+    if (row < 0) continue;
+    const int out_row = s.tiles_per_batch > 0 ? row : slot;
+    TO* dst = out + static_cast<int64_t>(out_row) * s.out_stride + batch * s.out_batch_step;
+    float weight = 1.f, lim = 0.f;
+    if constexpr (kGlu) {
+      weight = slot_weight ? slot_weight[slot] : 1.f;
+      lim = last ? s.limit_last : s.limit;
+    }
+#pragma unroll
+    for (int c = 0; c < (kGlu ? 2 : 4); ++c) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = o0 + (kGlu ? wave * 32 : wave * 64) + c * 16 + q * 4 + i;
+        if (o >= n_out) continue;
+        float y = acc[t][c][i];
+        if constexpr (kEpilogue == kGrSigmoidGate) {
+          const float g = bf16_to_f32(gate[static_cast<int64_t>(out_row) * s.gate_stride + batch * s.out_batch_step + o]);
+          y *= 1.f / (1.f + __expf(-g));
+        } else if constexpr (kGlu) {
+          const float a = fminf(y, lim);
+          const float b = fminf(fmaxf(acc[t][c + 2][i], -lim), lim);
+          y = weight * (a * (1.f / (1.f + __expf(-s.slope * a))) * (b + 1.f));
+        }
+        store_f32(dst + o, y);
+      }
+    }
+  }
+}
+
 // ---- the rows of every expert, side by side ------------------------------------------------------------------
 // chosen, weights [T, top]: the experts a row takes and its weights. Slots: every expert's rows together, an
 // expert's share padded to a multiple of `pad` (a tile's rows: 16 or 64), in expert order; then (with `shared`) all T rows once more for the
@@ -256,6 +387,9 @@ __global__ void __launch_bounds__(256) experts_sum_kernel(float* __restrict__ re
 
 using namespace alofa;
 
+// ALOFA_GROUPED_LDS=0 (read once; for measurements): tiles of 64 rows run without the LDS stage
+static const bool g_tiled = [] { const char* v = getenv("ALOFA_GROUPED_LDS"); return !(v && v[0] == '0'); }();
+
 template <int kEpilogue, typename TO>
 static int launch_grouped(void* out, const void* x, const void* W, const void* W2, const int32_t* tile_batch, const int32_t* row_in, const void* gate,
                           const float* slot_weight, const GroupedShape& s, int tile_rows, hipStream_t stream) {
@@ -271,7 +405,12 @@ static int launch_grouped(void* out, const void* x, const void* W, const void* W
   const unsigned grid = static_cast<unsigned>(shared_k ? tasks : (tasks + 3) / 4);
 #define ALOFA_GROUPED(RT, NC, KW) grouped_product_kernel<RT, NC, KW, kEpilogue, TO><<<grid, 256, 0, stream>>>(static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), \
     static_cast<const bf16_t*>(W2), tile_batch, row_in, static_cast<const bf16_t*>(gate), slot_weight, s, col_groups)
-  if (tile_rows == 64) ALOFA_GROUPED(4, 4, 1);
+  if (tile_rows == 64 && g_tiled) {
+    const int col_blocks = (widest + (kEpilogue == kGrClampedGlu ? 128 : 256) - 1) / (kEpilogue == kGrClampedGlu ? 128 : 256);
+    grouped_tiled_kernel<kEpilogue, TO><<<static_cast<unsigned>(s.tiles) * col_blocks, 256, 0, stream>>>(
+        static_cast<TO*>(out), static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(W), static_cast<const bf16_t*>(W2), tile_batch, row_in,
+        static_cast<const bf16_t*>(gate), slot_weight, s, col_blocks);
+  } else if (tile_rows == 64) ALOFA_GROUPED(4, 4, 1);
   else if (!shared_k) ALOFA_GROUPED(1, 4, 1);
   else if (nc == 2) ALOFA_GROUPED(1, 2, 4);
   else ALOFA_GROUPED(1, 1, 4);
