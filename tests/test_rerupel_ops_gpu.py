@@ -124,7 +124,7 @@ def test_gate_channel_scale_cap_and_squared_relu(dtype):
 
 
 @pytest.mark.parametrize("exact", [True, False])
-@pytest.mark.parametrize("experts, top", [(8, 3), (5, 5), (3, 1), (64, 6)])
+@pytest.mark.parametrize("experts, top", [(8, 3), (5, 5), (3, 1), (64, 6), (100, 7), (300, 2)])
 def test_the_choice_of_experts(experts, top, exact):
     from alofa_amd import ops
     rng = np.random.default_rng(experts)
