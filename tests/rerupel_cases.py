@@ -61,6 +61,14 @@ RERUPEL = {
     "F": _config(150, 64, 1e-6, 0.6, 25.0, 4.0, (89, 3, 11), (0, 2, 2), [
         (_latent(2, 16, 24, 264, 0.25), _dense(48)),
         (_latent(3, 32, 16, 320, 0.18), _moe(4, 2, 1.0, 16, 2.0, (16, 2.0)))]),
+    # five heads of 48 and 80 channels over a latent of 96; three layers passed through three times between two others; twelve experts of
+    # which a token takes three (slot by slot) or five (every expert against every row)
+    "G": _config(777, 320, 1e-5, 0.35, 15.0, 8.0, (1021, 17, 3), (1, 4, 3), [
+        (_latent(5, 48, 80, 96, 0.14), _dense(384)),
+        (_latent(5, 48, 80, 96, 0.14), _moe(12, 3, 1.7, 72, 1.2, (40, 1.2))),
+        (_latent(10, 32, 32, 160, 0.18), _moe(12, 5, 0.6, 72, 2.5, (72, 2.5))),
+        (_latent(5, 64, 64, 64, 0.125), _moe(12, 3, 1.7, 64, 1.2, (40, 1.2))),
+        (_latent(2, 128, 128, 192, 0.09), _dense(200))]),
 }
 
 
